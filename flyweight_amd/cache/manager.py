@@ -33,6 +33,20 @@ NO_PAGE = host.NO_PAGE
 _FIRST_NAMED_ID = 1 << 62       # ids of requests whose key is not a small non-negative integer
 
 
+def _flatten(path: Tuple, need: Mapping, flat: Dict) -> Dict:
+    """Every leaf of a nested mapping of needs into ``flat`` under the key path + names; returns
+    the mapping with those keys in place of the needs."""
+    names = {}
+    for name, below in need.items():
+        if isinstance(below, Mapping):
+            names[name] = _flatten(path + (name,), below, flat)
+        else:
+            names[name] = path + (name,)
+            if below is not None:
+                flat[path + (name,)] = below
+    return names
+
+
 class _Tables(Mapping):
     """The block tables of one page group: request -> page per block (NO_PAGE once given back)."""
 
@@ -116,7 +130,18 @@ class CacheManager:
         self.state_entries: Dict[int, CacheNeed] = {}
         self.needs: Dict[int, CacheNeed] = {}
         grouped: Dict[Tuple, Tuple[CacheNeed, List[int]]] = {}
-        for entry in sorted(needs):
+        # A mixer made of several (branches side by side, a recurrence with a convolution in front)
+        # asks for a mapping name -> need, nested at will: every leaf is a cache entry of its own,
+        # keyed (entry, name, ...), and the mixer sees the same mapping of views (``compound_view``).
+        self.compound: Dict[Hashable, Mapping] = {}
+        flat: Dict[Hashable, object] = {}
+        for entry, need in needs.items():
+            if isinstance(need, Mapping):
+                self.compound[entry] = _flatten(entry if isinstance(entry, tuple) else (entry,), need, flat)
+            else:
+                flat[entry] = need
+        needs = flat
+        for entry in sorted(needs, key=lambda key: key if isinstance(key, tuple) else (key,)):
             need = needs[entry]
             if need is None:
                 continue
@@ -192,6 +217,22 @@ class CacheManager:
     def view(self, entry: int, block_table=None, writes: bool = True):
         """What the mixer that uses cache entry ``entry`` sees of it."""
         return self.needs[entry].view(self.storage[entry], block_table, writes)
+
+    def compound_view(self, entry, block_tables: Sequence, writes: bool = True):
+        """For an entry whose need was a mapping: the same mapping with a view in place of every
+        need. ``block_tables``: this step's block-table rows of every page group."""
+        def build(names):
+            out = {}
+            for name, below in names.items():
+                if isinstance(below, Mapping):
+                    out[name] = build(below)
+                elif below in self.needs:
+                    group = self.entry_group.get(below)
+                    out[name] = self.view(below, None if group is None else block_tables[group], writes)
+                else:
+                    out[name] = None
+            return out
+        return build(self.compound[entry])
 
     # the tensors of the built-in needs, by entry
     @property

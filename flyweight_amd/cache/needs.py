@@ -78,14 +78,17 @@ class PagedKV(CacheNeed):
     num_kv_heads: int
     head_dim: int
     window: Optional[int] = None
+    v_head_dim: Optional[int] = None        # the size of a value where it is not the keys' (None: head_dim)
     paged = True
 
     def group_key(self) -> Tuple:
-        return ("kv", self.num_kv_heads, self.head_dim, self.window)
+        if self.v_head_dim in (None, self.head_dim):
+            return ("kv", self.num_kv_heads, self.head_dim, self.window)
+        return ("kv", self.num_kv_heads, self.head_dim, self.window, self.v_head_dim)
 
     def allocate(self, units, page_size, dtype, device):
         return (torch.zeros((units, self.num_kv_heads, page_size, self.head_dim), dtype=dtype, device=device),
-                torch.zeros((units, self.num_kv_heads, self.head_dim, page_size), dtype=dtype, device=device))
+                torch.zeros((units, self.num_kv_heads, self.v_head_dim or self.head_dim, page_size), dtype=dtype, device=device))
 
     def view(self, storage, block_table, writes):
         return CacheView(k_pages=storage[0], v_pages=storage[1], block_table=block_table, writes=writes)

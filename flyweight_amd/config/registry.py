@@ -36,13 +36,13 @@ def architecture_name(data: Mapping[str, Any]) -> str:
     names = data.get("architectures")
     if isinstance(names, list) and names and isinstance(names[0], str):
         return names[0]
-    model_type = data.get("model_type")
-    if isinstance(model_type, str):
-        return model_type
-    raise ConfigError("config.json is missing 'architectures' (and 'model_type')")
+    for key in ("model_type", "architecture"):      # some layouts name their one architecture in a string
+        if isinstance(data.get(key), str):
+            return data[key]
+    raise ConfigError("config.json is missing 'architectures' (and 'model_type', 'architecture')")
 
 
-def config_from_dict(data: Mapping[str, Any]):
+def config_class_of(data: Mapping[str, Any]):
     if not isinstance(data, Mapping):
         raise ConfigError("config.json must hold a JSON object")
     name = architecture_name(data)
@@ -52,7 +52,11 @@ def config_from_dict(data: Mapping[str, Any]):
     if config_class is None:
         raise ConfigError(
             f"unknown architecture '{name}'; registered: {', '.join(registered_architectures()) or 'none'}")
-    return config_class.from_dict(data)
+    return config_class
+
+
+def config_from_dict(data: Mapping[str, Any]):
+    return config_class_of(data).from_dict(data)
 
 
 def load_config(model_dir: str):
@@ -63,4 +67,7 @@ def load_config(model_dir: str):
         data = json_reader.parse_file(path)
     except json_reader.JsonError as error:
         raise ConfigError(f"{path}: {error}") from None
-    return config_from_dict(data)
+    config_class = config_class_of(data)
+    if hasattr(config_class, "from_model_dir"):     # sizes that only the checkpoint's tensor shapes show
+        return config_class.from_model_dir(model_dir, data)
+    return config_class.from_dict(data)

@@ -43,13 +43,16 @@ class PartSpec:
 
 @dataclass(frozen=True)
 class LayerSpec:
-    """A residual block: which arrangement, and the four parts it is made of."""
+    """A residual block: which arrangement, and the four parts it is made of (an arrangement may
+    allow a layer without a feed-forward: ``ffn`` and ``ffn_norm`` None). ``params``: constants of
+    the arrangement itself (a factor on what joins the residual stream, for instance)."""
 
     arrangement: str            # key into the block registry, e.g. "pre_norm_residual"
     mixer_norm: PartSpec
     mixer: PartSpec
-    ffn_norm: PartSpec
-    ffn: PartSpec
+    ffn_norm: Optional[PartSpec]
+    ffn: Optional[PartSpec]
+    params: Mapping[str, Any] = field(default_factory=dict)
 
 
 @dataclass(frozen=True)

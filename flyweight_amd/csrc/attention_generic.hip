@@ -12,8 +12,8 @@
 #define ATTN_PAGE 64
 #define ATTN_MAX_HEAD_DIM 256
 
-// One wave per (row, head-vector). Head-vectors 0..nh-1 are queries, nh..nh+nkv-1 keys,
-// the rest values. Per-head RMS norm then half-split rotation: channel i pairs with
+// One wave per (row, head-vector). Head-vectors 0..nh-1 are queries, nh..nh+nkv-1 keys (head_dim
+// channels each), the rest values (v_dim channels each, which may differ from head_dim). Per-head RMS norm then half-split rotation: channel i pairs with
 // i + rotary_dim/2; out[i] = a cos - b sin, out[i + half] = b cos + a sin
 // (native/include/flyweight_v2_native_kernels.hpp:1015-1050). Values are stored untouched.
 template <typename TI, typename T>
@@ -22,21 +22,23 @@ __global__ __launch_bounds__(64) void qk_norm_rope_kv_write_kernel(
     const float* __restrict__ k_norm_weight, float eps, const float* __restrict__ cos_table,
     const float* __restrict__ sin_table, int rotary_dim, T* __restrict__ k_pages, T* __restrict__ v_pages,
     const int32_t* __restrict__ block_table, int table_stride, const int32_t* __restrict__ row_seg,
-    const int32_t* __restrict__ row_pos, int num_heads, int num_kv_heads, int head_dim) {
+    const int32_t* __restrict__ row_pos, int num_heads, int num_kv_heads, int head_dim, int v_dim) {
     __shared__ float normed[ATTN_MAX_HEAD_DIM];
     const int row = blockIdx.x;
     const int vec = blockIdx.y;
     const int lane = threadIdx.x;
-    const int width = (num_heads + 2 * num_kv_heads) * head_dim;
-    const TI* source = qkv + (size_t)row * width + (size_t)vec * head_dim;
+    const int width = (num_heads + num_kv_heads) * head_dim + num_kv_heads * v_dim;
+    const TI* source = qkv + (size_t)row * width + (vec < num_heads + num_kv_heads
+                           ? (size_t)vec * head_dim
+                           : (size_t)(num_heads + num_kv_heads) * head_dim + (size_t)(vec - num_heads - num_kv_heads) * v_dim);
     const int pos = row_pos[row];
     const int page = block_table[(size_t)row_seg[row] * table_stride + pos / ATTN_PAGE];
     const int slot = pos % ATTN_PAGE;
 
     if (vec >= num_heads + num_kv_heads) {      // value head: transposed store
         const int kvh = vec - num_heads - num_kv_heads;
-        T* dest = v_pages + ((size_t)page * num_kv_heads + kvh) * head_dim * ATTN_PAGE;
-        for (int d = lane; d < head_dim; d += 64) store_from_float(dest, (size_t)d * ATTN_PAGE + slot, load_as_float(source, d));
+        T* dest = v_pages + ((size_t)page * num_kv_heads + kvh) * v_dim * ATTN_PAGE;
+        for (int d = lane; d < v_dim; d += 64) store_from_float(dest, (size_t)d * ATTN_PAGE + slot, load_as_float(source, d));
         return;
     }
     const bool is_query = vec < num_heads;
@@ -164,9 +166,10 @@ extern "C" int fw_qk_norm_rope_kv_write(const void* qkv, int in_dtype, void* q_o
                                         const float* sin_table, int rotary_dim, void* k_pages, void* v_pages,
                                         const int32_t* block_table, int table_stride, const int32_t* row_seg,
                                         const int32_t* row_pos, int rows, int num_heads, int num_kv_heads,
-                                        int head_dim, int page_size, int num_pages, int write_kv, void* stream) {
+                                        int head_dim, int v_dim, int page_size, int num_pages, int write_kv, void* stream) {
     FW_REQUIRE(rows >= 0 && num_heads > 0 && num_kv_heads > 0, "qk_norm_rope: bad sizes rows=%d heads=%d kv_heads=%d", rows, num_heads, num_kv_heads);
     FW_REQUIRE(head_dim > 0 && head_dim <= ATTN_MAX_HEAD_DIM, "qk_norm_rope: head_dim %d outside 1..%d", head_dim, ATTN_MAX_HEAD_DIM);
+    FW_REQUIRE(v_dim > 0 && v_dim <= ATTN_MAX_HEAD_DIM, "qk_norm_rope: value size %d outside 1..%d", v_dim, ATTN_MAX_HEAD_DIM);
     FW_REQUIRE(rotary_dim >= 0 && rotary_dim <= head_dim && rotary_dim % 2 == 0, "qk_norm_rope: rotary_dim %d must be even and at most head_dim %d", rotary_dim, head_dim);
     FW_REQUIRE(rotary_dim == 0 || (cos_table && sin_table), "qk_norm_rope: rotation asked for without tables");
     FW_REQUIRE(page_size == ATTN_PAGE, "qk_norm_rope: page size must be %d, got %d", ATTN_PAGE, page_size);
@@ -178,7 +181,7 @@ extern "C" int fw_qk_norm_rope_kv_write(const void* qkv, int in_dtype, void* q_o
     FW_REQUIRE(vectors <= 65535, "qk_norm_rope: too many heads (%d)", vectors);
     dim3 grid(rows, vectors);
     hipStream_t s = (hipStream_t)stream;
-    if (head_dim <= 64 && rows >= 8 * QK_ROWS) {    // a prompt's rows, eight to a wave
+    if (head_dim <= 64 && v_dim == head_dim && rows >= 8 * QK_ROWS) {    // a prompt's rows, eight to a wave
         dim3 by_rows((rows + QK_ROWS - 1) / QK_ROWS, vectors);
 #define FW_QK_ROWS_LAUNCH(TI, T)                                                                                     \
     qk_norm_rope_kv_write_rows_kernel<TI, T><<<by_rows, 64, 0, s>>>(                                                 \
@@ -195,7 +198,7 @@ extern "C" int fw_qk_norm_rope_kv_write(const void* qkv, int in_dtype, void* q_o
 #define FW_QK_LAUNCH(TI, T)                                                                                          \
     qk_norm_rope_kv_write_kernel<TI, T><<<grid, 64, 0, s>>>(                                                         \
         (const TI*)qkv, (T*)q_out, q_norm_weight, k_norm_weight, eps, cos_table, sin_table, rotary_dim, (T*)k_pages, \
-        (T*)v_pages, block_table, table_stride, row_seg, row_pos, num_heads, num_kv_heads, head_dim)
+        (T*)v_pages, block_table, table_stride, row_seg, row_pos, num_heads, num_kv_heads, head_dim, v_dim)
     if (in_dtype == FW_F32 && dtype == FW_F32) FW_QK_LAUNCH(float, float);
     else if (in_dtype == FW_F32 && dtype == FW_BF16) FW_QK_LAUNCH(float, bf16_t);
     else if (in_dtype == FW_BF16 && dtype == FW_BF16) FW_QK_LAUNCH(bf16_t, bf16_t);
@@ -214,7 +217,7 @@ template <typename T>
 __global__ __launch_bounds__(64) void attention_generic_kernel(
     const T* __restrict__ q, T* __restrict__ out, const T* __restrict__ k_pages, const T* __restrict__ v_pages,
     const int32_t* __restrict__ block_table, int table_stride, const int32_t* __restrict__ row_seg,
-    const int32_t* __restrict__ row_pos, int num_heads, int num_kv_heads, int head_dim, float scale, int window) {
+    const int32_t* __restrict__ row_pos, int num_heads, int num_kv_heads, int head_dim, int v_dim, float scale, int window) {
     __shared__ float qs[ATTN_MAX_HEAD_DIM];
     __shared__ float ps[ATTN_PAGE];
     const int row = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
@@ -250,8 +253,8 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
 #pragma unroll
         for (int j = 0; j < ATTN_MAX_HEAD_DIM / 64; ++j) {
             const int d = lane + 64 * j;
-            if (d < head_dim) {
-                const T* value = v_pages + (((size_t)page * num_kv_heads + kvh) * head_dim + d) * ATTN_PAGE;
+            if (d < v_dim) {
+                const T* value = v_pages + (((size_t)page * num_kv_heads + kvh) * v_dim + d) * ATTN_PAGE;
                 float sum = 0.0f;
                 for (int s = lo; s <= hi; ++s) sum = fmaf(ps[s], load_as_float(value, s), sum);
                 acc[j] = acc[j] * alpha + sum;
@@ -259,19 +262,20 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
         }
         __syncthreads();
     }
-    T* dest = out + ((size_t)row * num_heads + head) * head_dim;
+    T* dest = out + ((size_t)row * num_heads + head) * v_dim;
 #pragma unroll
     for (int j = 0; j < ATTN_MAX_HEAD_DIM / 64; ++j) {
         const int d = lane + 64 * j;
-        if (d < head_dim) store_from_float(dest, d, acc[j] / running_sum);
+        if (d < v_dim) store_from_float(dest, d, acc[j] / running_sum);
     }
 }
 
 extern "C" int fw_attention_generic(const void* q, void* out, int dtype, const void* k_pages,
                                     const void* v_pages, const int32_t* block_table, int table_stride,
                                     const int32_t* row_seg, const int32_t* row_pos, int rows, int num_heads,
-                                    int num_kv_heads, int head_dim, float scale, int window, int page_size,
+                                    int num_kv_heads, int head_dim, int v_dim, float scale, int window, int page_size,
                                     int num_pages, void* stream) {
+    FW_REQUIRE(v_dim > 0 && v_dim <= ATTN_MAX_HEAD_DIM, "attention: value size %d outside 1..%d", v_dim, ATTN_MAX_HEAD_DIM);
     FW_REQUIRE(rows >= 0 && num_heads > 0 && num_kv_heads > 0 && num_heads % num_kv_heads == 0,
                "attention: heads %d must be a positive multiple of kv heads %d", num_heads, num_kv_heads);
     FW_REQUIRE(head_dim > 0 && head_dim <= ATTN_MAX_HEAD_DIM, "attention: head_dim %d outside 1..%d", head_dim, ATTN_MAX_HEAD_DIM);
@@ -284,11 +288,11 @@ extern "C" int fw_attention_generic(const void* q, void* out, int dtype, const v
     if (dtype == FW_F32)
         attention_generic_kernel<float><<<grid, 64, 0, (hipStream_t)stream>>>(
             (const float*)q, (float*)out, (const float*)k_pages, (const float*)v_pages, block_table, table_stride,
-            row_seg, row_pos, num_heads, num_kv_heads, head_dim, scale, window);
+            row_seg, row_pos, num_heads, num_kv_heads, head_dim, v_dim, scale, window);
     else if (dtype == FW_BF16)
         attention_generic_kernel<bf16_t><<<grid, 64, 0, (hipStream_t)stream>>>(
             (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)k_pages, (const bf16_t*)v_pages, block_table, table_stride,
-            row_seg, row_pos, num_heads, num_kv_heads, head_dim, scale, window);
+            row_seg, row_pos, num_heads, num_kv_heads, head_dim, v_dim, scale, window);
     else
         FW_REQUIRE(false, "attention: unknown dtype %d", dtype);
     FW_LAUNCH_CHECK("attention_generic");

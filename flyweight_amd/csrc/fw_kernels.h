@@ -120,21 +120,21 @@ int fw_shortconv(const void* bcx, int in_dtype, void* out, int out_dtype, const 
 
 // Per-head RMS norm of q and k (weights may be null: no norm), half-split rotation of the
 // first rotary_dim channels by the row's angle, q out, k and v appended to the pages of
-// the row's segment. qkv [rows][(nh + 2 nkv) hd]. k_pages [pages][nkv][P][hd];
-// v_pages [pages][nkv][hd][P]. block_table [segments][table_stride].
+// the row's segment. qkv [rows][(nh + nkv) hd + nkv vd]: values may have a size vd of their own.
+// k_pages [pages][nkv][P][hd]; v_pages [pages][nkv][vd][P]. block_table [segments][table_stride].
 int fw_qk_norm_rope_kv_write(const void* qkv, int in_dtype, void* q_out, int dtype, const float* q_norm_weight,
                              const float* k_norm_weight, float eps, const float* cos_table,
                              const float* sin_table, int rotary_dim, void* k_pages, void* v_pages,
                              const int32_t* block_table, int table_stride, const int32_t* row_seg,
                              const int32_t* row_pos, int rows, int num_heads, int num_kv_heads,
-                             int head_dim, int page_size, int num_pages, int write_kv, void* stream);
+                             int head_dim, int v_dim, int page_size, int num_pages, int write_kv, void* stream);
 
 // Causal attention of every row over the cached keys 0..row_pos[r] (or the last `window`
-// of them) of its segment. out [rows][nh*hd].
+// of them) of its segment. out [rows][nh*vd].
 int fw_attention_generic(const void* q, void* out, int dtype, const void* k_pages,
                          const void* v_pages, const int32_t* block_table, int table_stride,
                          const int32_t* row_seg, const int32_t* row_pos, int rows, int num_heads,
-                         int num_kv_heads, int head_dim, float scale, int window, int page_size,
+                         int num_kv_heads, int head_dim, int v_dim, float scale, int window, int page_size,
                          int num_pages, void* stream);
 
 // The same attention on the matrix cores, bfloat16 only, head_dim a multiple of 16 up to 256.
@@ -200,6 +200,43 @@ int fw_sample_rows(const float* logits, const float* settings, unsigned long lon
 int fw_fill_zero(void* ptr, long long bytes, void* stream);
 // `pieces` runs of `bytes` each, `stride_bytes` apart, cleared in one launch
 int fw_fill_zero_pieces(void* ptr, int pieces, long long bytes, long long stride_bytes, void* stream);
+
+// ---- the gated delta rule (a linear recurrence over a matrix state per head) -----------------------
+// What the recurrence reads, from one step's projections. proj [rows][proj_stride]: columns
+// 0 .. 2 G d + H vd - 1 hold q | k | v before their short causal convolutions (G = kv_heads heads of d
+// = dim channels for q and for k, H = heads of vd = vdim channels for v), columns beta_col .. + H - 1
+// the write strengths before their sigmoid. a [rows][H d]: the decays' arguments. taps [channels][L],
+// the last column the current token's; conv_state [slots][channels][L - 1], oldest first, read and
+// then moved on by the segment's rows. qkv_out [rows][channels]: silu of the convolutions, q and k of
+// unit length per head (sum of squares + 1e-6 under the root), q also times d^-1/2. decay_out
+// [rows][H d] = exp(-exp(A_log[h]) * softplus(a + dt_bias)); beta_out [rows][H].
+int fw_delta_prepare(const void* proj, int dtype, int proj_stride, int beta_col, const void* a, const float* taps,
+                     float* conv_state, const float* A_log, const float* dt_bias, const int32_t* row_seg,
+                     const int32_t* seg_row0, const int32_t* seg_slot, float* qkv_out, float* decay_out,
+                     float* beta_out, int rows, int segments, int heads, int kv_heads, int dim, int vdim,
+                     int taps_count, int slots, void* stream);
+// Per segment and head, token by token: S <- diag(g) S; u = beta (v - S^T k); S <- S + k u^T;
+// o = S^T q. state [slots][H][vd][d] (S transposed), read at the segment's start and written at its
+// end. out [rows][H vd]. Head h reads q/k head h / (H / G).
+int fw_gated_delta_rule(const float* qkv, const float* decay, const float* beta, float* state, float* out,
+                        const int32_t* seg_row0, const int32_t* seg_slot, int rows, int segments, int heads,
+                        int kv_heads, int dim, int vdim, int slots, void* stream);
+// out[r][h][j] = o[r][h][j] * rsqrt(mean_j o[r][h]^2 + eps) * weight[j] * sigmoid(gate[r][h vd + j])
+int fw_gated_head_norm(const float* o, const void* gate, int gate_dtype, int gate_stride, const float* weight,
+                       void* out, int out_dtype, int rows, int heads, int vdim, float eps, void* stream);
+
+// ---- sublayers whose output is normed ------------------------------------------------------------
+// x[r] += mult * rmsnorm(scale_a a[r] + scale_b b[r]) * w (b may be null; one_centered: 1 + w);
+// rounded (may be null): the new x once more in rounded_dtype, for the products that read it next.
+int fw_norm_scale_add(float* x, const float* a, const float* b, float scale_a, float scale_b, const float* weight,
+                      int one_centered, float eps, float mult, void* rounded, int rounded_dtype, int rows,
+                      int hidden, void* stream);
+// out (bfloat16) = x (float32), count elements
+int fw_round_rows(const float* x, void* out, long long count, void* stream);
+// gate_up [rows][2 I]: out[r][i] = g sigmoid(alpha g) (u + shift), g = min(gate, limit),
+// u = clamp(up, -limit, limit)
+int fw_clamped_glu(const void* gate_up, int in_dtype, void* out, int out_dtype, int rows, int intermediate,
+                   float limit, float alpha, float shift, void* stream);
 
 #ifdef __cplusplus
 }

@@ -1,0 +1,139 @@
+// What stands around a sublayer whose OUTPUT is normed before it joins the residual stream:
+//     x <- x + mult * rmsnorm(scale_a * a + scale_b * b) * w
+// (b optional: two branches that read the same input and are mixed with fixed weights), the rounded
+// copy of the new x that the next sublayer's products read, and a gated linear unit with clamped
+// halves. Sums and the residual stream are float32.
+#include "fw_common.h"
+#include "fw_kernels.h"
+
+__device__ __forceinline__ float sublayer_sigmoid(float g) {
+    if (g >= 0.0f) return 1.0f / (1.0f + expf(-g));
+    const float e = expf(g);
+    return e / (1.0f + e);
+}
+
+// One workgroup per row. y = scale_a a (+ scale_b b) is formed once and kept in registers (rows of up
+// to 256 * NORM_ADD_HELD channels) or formed again in the second pass (wider rows).
+#define NORM_ADD_HELD 16
+template <typename T>
+__global__ __launch_bounds__(256) void norm_scale_add_kernel(
+    float* __restrict__ x, const float* __restrict__ a, const float* __restrict__ b, float scale_a, float scale_b,
+    const float* __restrict__ weight, int one_centered, float eps, float mult, T* __restrict__ rounded, int hidden) {
+    __shared__ float scratch[16];
+    const size_t row0 = (size_t)blockIdx.x * hidden;
+    const bool held_all = hidden <= 256 * NORM_ADD_HELD;
+    float held[NORM_ADD_HELD];
+    float sum = 0.0f;
+    if (held_all) {
+#pragma unroll
+        for (int u = 0; u < NORM_ADD_HELD; ++u) {
+            const int i = threadIdx.x + 256 * u;
+            float y = 0.0f;
+            if (i < hidden) {
+                y = scale_a * a[row0 + i];
+                if (b) y = fmaf(scale_b, b[row0 + i], y);
+            }
+            held[u] = y;
+            sum = fmaf(y, y, sum);
+        }
+    } else {
+        for (int i = threadIdx.x; i < hidden; i += 256) {
+            float y = scale_a * a[row0 + i];
+            if (b) y = fmaf(scale_b, b[row0 + i], y);
+            sum = fmaf(y, y, sum);
+        }
+    }
+    sum = block_sum(sum, scratch);
+    const float inv = 1.0f / sqrtf(sum / (float)hidden + eps);
+    const float one = one_centered ? 1.0f : 0.0f;
+    if (held_all) {
+#pragma unroll
+        for (int u = 0; u < NORM_ADD_HELD; ++u) {
+            const int i = threadIdx.x + 256 * u;
+            if (i < hidden) {
+                const float updated = x[row0 + i] + mult * (held[u] * inv * (weight[i] + one));
+                x[row0 + i] = updated;
+                if (rounded) store_from_float(rounded, row0 + i, updated);
+            }
+        }
+    } else {
+        for (int i = threadIdx.x; i < hidden; i += 256) {
+            float y = scale_a * a[row0 + i];
+            if (b) y = fmaf(scale_b, b[row0 + i], y);
+            const float updated = x[row0 + i] + mult * (y * inv * (weight[i] + one));
+            x[row0 + i] = updated;
+            if (rounded) store_from_float(rounded, row0 + i, updated);
+        }
+    }
+}
+
+extern "C" int fw_norm_scale_add(float* x, const float* a, const float* b, float scale_a, float scale_b, const float* weight,
+                                 int one_centered, float eps, float mult, void* rounded, int rounded_dtype, int rows,
+                                 int hidden, void* stream) {
+    FW_REQUIRE(rows >= 0 && hidden > 0, "norm_scale_add: bad sizes rows=%d hidden=%d", rows, hidden);
+    FW_REQUIRE(eps > 0.0f, "norm_scale_add: eps must be positive");
+    FW_REQUIRE(x && a && weight, "norm_scale_add: x, a and the weight are needed");
+    if (rows == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    if (!rounded || rounded_dtype == FW_F32)
+        norm_scale_add_kernel<float><<<rows, 256, 0, s>>>(x, a, b, scale_a, scale_b, weight, one_centered, eps, mult, (float*)rounded, hidden);
+    else if (rounded_dtype == FW_BF16)
+        norm_scale_add_kernel<bf16_t><<<rows, 256, 0, s>>>(x, a, b, scale_a, scale_b, weight, one_centered, eps, mult, (bf16_t*)rounded, hidden);
+    else
+        FW_REQUIRE(false, "norm_scale_add: unknown dtype %d", rounded_dtype);
+    FW_LAUNCH_CHECK("norm_scale_add");
+    return 0;
+}
+
+// float32 rows rounded to the activation type
+__global__ void round_rows_kernel(const float* __restrict__ x, bf16_t* __restrict__ out, long long count) {
+    for (long long i = blockIdx.x * (long long)blockDim.x + threadIdx.x; i < count; i += (long long)gridDim.x * blockDim.x)
+        out[i] = float_to_bf16(x[i]);
+}
+
+extern "C" int fw_round_rows(const float* x, void* out, long long count, void* stream) {
+    FW_REQUIRE(count >= 0, "round_rows: negative count");
+    if (count == 0) return 0;
+    const int blocks = (int)((count + 255) / 256 < 4096 ? (count + 255) / 256 : 4096);
+    round_rows_kernel<<<blocks, 256, 0, (hipStream_t)stream>>>(x, (bf16_t*)out, count);
+    FW_LAUNCH_CHECK("round_rows");
+    return 0;
+}
+
+// Gated linear unit with clamped halves: g = min(gate, limit), u = clamp(up, -limit, limit),
+// out = g * sigmoid(alpha * g) * (u + shift). gate_up [rows][2 I]: gate columns, then up columns.
+template <typename TI, typename TO>
+__global__ void clamped_glu_kernel(const TI* __restrict__ gate_up, TO* __restrict__ out, int intermediate, float limit,
+                                   float alpha, float shift) {
+    const int row = blockIdx.y;
+    const TI* source = gate_up + (size_t)row * 2 * intermediate;
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < intermediate; i += gridDim.x * blockDim.x) {
+        const float g = fminf(load_as_float(source, i), limit);
+        const float u = fminf(fmaxf(load_as_float(source, (size_t)intermediate + i), -limit), limit);
+        store_from_float(out, (size_t)row * intermediate + i, g * sublayer_sigmoid(alpha * g) * (u + shift));
+    }
+}
+
+extern "C" int fw_clamped_glu(const void* gate_up, int in_dtype, void* out, int out_dtype, int rows, int intermediate,
+                              float limit, float alpha, float shift, void* stream) {
+    FW_REQUIRE(rows >= 0 && rows <= 65535 * 16 && intermediate > 0, "clamped_glu: bad sizes rows=%d intermediate=%d", rows, intermediate);
+    FW_REQUIRE(limit > 0.0f, "clamped_glu: the limit must be positive");
+    if (rows == 0) return 0;
+    int across = (intermediate + 255) / 256;
+    if (across > 64) across = 64;
+    hipStream_t s = (hipStream_t)stream;
+    for (int row0 = 0; row0 < rows; row0 += 65535) {
+        const int now = rows - row0 < 65535 ? rows - row0 : 65535;
+        dim3 grid(across, now);
+        const size_t in_at = (size_t)row0 * 2 * intermediate, out_at = (size_t)row0 * intermediate;
+#define FW_GLU_LAUNCH(TI, TO) \
+    clamped_glu_kernel<TI, TO><<<grid, 256, 0, s>>>((const TI*)gate_up + in_at, (TO*)out + out_at, intermediate, limit, alpha, shift)
+        if (in_dtype == FW_F32 && out_dtype == FW_F32) FW_GLU_LAUNCH(float, float);
+        else if (in_dtype == FW_F32 && out_dtype == FW_BF16) FW_GLU_LAUNCH(float, bf16_t);
+        else if (in_dtype == FW_BF16 && out_dtype == FW_BF16) FW_GLU_LAUNCH(bf16_t, bf16_t);
+        else FW_REQUIRE(false, "clamped_glu: unsupported dtypes in=%d out=%d", in_dtype, out_dtype);
+#undef FW_GLU_LAUNCH
+    }
+    FW_LAUNCH_CHECK("clamped_glu");
+    return 0;
+}

@@ -73,6 +73,8 @@ class Model:
 
 
 class Runtime:
+    LARGEST_DEFAULT_CONTEXT = 1 << 17       # the context limit taken when neither the caller nor the model gives one
+
     def __init__(self, model: Model, context_limit: Optional[int] = None, parallel_sequences: int = 16,
                  num_pages: Optional[int] = None, max_batch_tokens: int = 2048, prefill_rows: int = 512,
                  decode_steps_per_turn: int = 1):
@@ -88,6 +90,10 @@ class Runtime:
         self.model = model
         spec = model.spec
         self.context_limit = min(context_limit or spec.max_positions, spec.max_positions)
+        if not context_limit and self.context_limit > self.LARGEST_DEFAULT_CONTEXT:
+            # a model that sets no limit of its own (positions enter through angles and recurrences only):
+            # what the given pages hold, or a default; block tables and pools are sized by this
+            self.context_limit = min(self.context_limit, int(num_pages) * PAGE_SIZE if num_pages else self.LARGEST_DEFAULT_CONTEXT)
         self.parallel_sequences = max(1, int(parallel_sequences))
         per_request = (self.context_limit + PAGE_SIZE - 1) // PAGE_SIZE
         self.num_pages = int(num_pages) if num_pages else per_request * self.parallel_sequences

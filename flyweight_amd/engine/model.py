@@ -88,11 +88,17 @@ class CausalLM:
         """The parts that ask for index arrays of their own in every step's upload
         (``Part.step_arrays``), one for each distinct key."""
         found: Dict = {}
+
+        def visit(part) -> None:
+            key = part.step_arrays_key()
+            if key is not None:
+                found.setdefault(key, part)
+            for below in (part.sub_parts() if hasattr(part, "sub_parts") else ()):     # a part made of parts
+                visit(below)
+
         for block in self.layers:
             for part in block.parts():
-                key = part.step_arrays_key()
-                if key is not None:
-                    found.setdefault(key, part)
+                visit(part)
         return list(found.values())
 
     # ----- forward ----------------------------------------------------------------------

@@ -363,6 +363,8 @@ class StepContext:
     def cache_view(self, cache: CacheManager, entry):
         """What the mixer of schedule entry ``entry`` sees of the cache: the view its need class
         gives of the entry's storage (with this step's block-table rows, for a paged one)."""
+        if entry.cache is not None and entry.cache in cache.compound:
+            return cache.compound_view(entry.cache, self.block_tables, entry.writes_cache)
         if entry.cache is None or entry.cache not in cache.needs:
             return CacheView(writes=False if entry.cache is None else entry.writes_cache)
         group = cache.entry_group.get(entry.cache)

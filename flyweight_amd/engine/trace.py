@@ -47,7 +47,8 @@ def replay(model_dir: str, dtype: str, out_dir: str, max_tokens: int, lines: IO[
     os.makedirs(out_dir, exist_ok=True)
     _, model = load_model(model_dir, dtype=dtype, device=device)
     num_pages = (max_tokens + PAGE_SIZE - 1) // PAGE_SIZE
-    stepper = Stepper(model, num_pages=num_pages, max_requests=min(num_pages, MAX_LIVE_SLOTS), page_size=PAGE_SIZE)
+    stepper = Stepper(model, num_pages=num_pages, max_requests=min(num_pages, MAX_LIVE_SLOTS), page_size=PAGE_SIZE,
+                      context_limit=min(model.spec.max_positions, num_pages * PAGE_SIZE))
     for number, line in enumerate(lines):
         line = line.strip()
         if not line:

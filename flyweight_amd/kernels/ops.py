@@ -19,7 +19,7 @@ from . import build as _build
 F32, BF16 = 0, 1
 PAGE_SIZE = 64          # tokens per cache page: the width of a wavefront
 MAX_HEAD_DIM = 256
-ABI_VERSION = 9
+ABI_VERSION = 10
 
 _lib = None
 
@@ -303,12 +303,14 @@ def shortconv(bcx: torch.Tensor, taps: torch.Tensor, conv_bias: Optional[torch.T
     return out
 
 
-def _check_pages(k_pages: torch.Tensor, v_pages: torch.Tensor, kv_heads: int, head_dim: int, dtype: torch.dtype):
+def _check_pages(k_pages: torch.Tensor, v_pages: torch.Tensor, kv_heads: int, head_dim: int, dtype: torch.dtype,
+                 v_dim: Optional[int] = None):
     pages = k_pages.shape[0]
+    v_dim = head_dim if v_dim is None else v_dim
     if k_pages.shape != (pages, kv_heads, PAGE_SIZE, head_dim):
         raise KernelError(f"K pages are {tuple(k_pages.shape)}, expected [pages, {kv_heads}, {PAGE_SIZE}, {head_dim}]")
-    if v_pages.shape != (pages, kv_heads, head_dim, PAGE_SIZE):
-        raise KernelError(f"V pages are {tuple(v_pages.shape)}, expected [pages, {kv_heads}, {head_dim}, {PAGE_SIZE}]")
+    if v_pages.shape != (pages, kv_heads, v_dim, PAGE_SIZE):
+        raise KernelError(f"V pages are {tuple(v_pages.shape)}, expected [pages, {kv_heads}, {v_dim}, {PAGE_SIZE}]")
     if k_pages.dtype != dtype or v_pages.dtype != dtype:
         raise KernelError(f"cache pages are {k_pages.dtype}/{v_pages.dtype} but activations are {dtype}")
     return pages
@@ -318,13 +320,16 @@ def qk_norm_rope_kv_write(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, 
                           q_norm_weight: Optional[torch.Tensor], k_norm_weight: Optional[torch.Tensor], eps: float,
                           cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], rotary_dim: int,
                           k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,
-                          row_seg: torch.Tensor, row_pos: torch.Tensor, write_kv: bool = True) -> torch.Tensor:
-    """The output and the cache take the pages' dtype; ``qkv`` may be float32 beside bfloat16 pages."""
+                          row_seg: torch.Tensor, row_pos: torch.Tensor, write_kv: bool = True,
+                          v_dim: Optional[int] = None) -> torch.Tensor:
+    """The output and the cache take the pages' dtype; ``qkv`` may be float32 beside bfloat16 pages.
+    ``v_dim``: the size of a value head where it is not ``head_dim``."""
     _dev(qkv, q_norm_weight, k_norm_weight, cos, sin, k_pages, v_pages, block_table, row_seg, row_pos)
     rows, width = qkv.shape
-    if width != (num_heads + 2 * num_kv_heads) * head_dim:
-        raise KernelError(f"qk_norm_rope: qkv width {width} != ({num_heads} + 2 x {num_kv_heads}) x {head_dim}")
-    pages = _check_pages(k_pages, v_pages, num_kv_heads, head_dim, k_pages.dtype)
+    v_dim = head_dim if v_dim is None else int(v_dim)
+    if width != (num_heads + num_kv_heads) * head_dim + num_kv_heads * v_dim:
+        raise KernelError(f"qk_norm_rope: qkv width {width} != ({num_heads} + {num_kv_heads}) x {head_dim} + {num_kv_heads} x {v_dim}")
+    pages = _check_pages(k_pages, v_pages, num_kv_heads, head_dim, k_pages.dtype, v_dim)
     for w in (q_norm_weight, k_norm_weight):
         if w is not None:
             _want(w, torch.float32, "norm weight")
@@ -344,27 +349,29 @@ def qk_norm_rope_kv_write(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, 
     _check(library().fw_qk_norm_rope_kv_write(
         _p(qkv), _code(qkv.dtype), _p(q_out), _code(k_pages.dtype), _p(q_norm_weight), _p(k_norm_weight), ctypes.c_float(eps), _p(cos), _p(sin),
         rotary_dim, _p(k_pages), _p(v_pages), _p(block_table), block_table.shape[1], _p(row_seg), _p(row_pos), rows,
-        num_heads, num_kv_heads, head_dim, PAGE_SIZE, pages, int(write_kv), _stream()))
+        num_heads, num_kv_heads, head_dim, v_dim, PAGE_SIZE, pages, int(write_kv), _stream()))
     return q_out
 
 
 def attention_generic(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, k_pages: torch.Tensor,
                       v_pages: torch.Tensor, block_table: torch.Tensor, row_seg: torch.Tensor, row_pos: torch.Tensor,
-                      scale: float, window: int = 0) -> torch.Tensor:
+                      scale: float, window: int = 0, v_dim: Optional[int] = None) -> torch.Tensor:
+    """``v_dim``: the size of a value head (and of a head's output) where it is not ``head_dim``."""
     _dev(q, k_pages, v_pages, block_table, row_seg, row_pos)
     rows = q.shape[0]
+    v_dim = head_dim if v_dim is None else int(v_dim)
     if q.shape != (rows, num_heads * head_dim):
         raise KernelError(f"attention: q is {tuple(q.shape)}, expected {(rows, num_heads * head_dim)}")
-    pages = _check_pages(k_pages, v_pages, num_kv_heads, head_dim, q.dtype)
+    pages = _check_pages(k_pages, v_pages, num_kv_heads, head_dim, q.dtype, v_dim)
     _want(block_table, torch.int32, "block_table")
     _want(row_seg, torch.int32, "row_seg")
     _want(row_pos, torch.int32, "row_pos")
     if block_table.dim() != 2 or row_seg.numel() < rows or row_pos.numel() < rows:
         raise KernelError("attention: batch index arrays are too short")
-    out = torch.empty_like(q)
+    out = torch.empty((rows, num_heads * v_dim), dtype=q.dtype, device=q.device)
     _check(library().fw_attention_generic(
         _p(q), _p(out), _code(q.dtype), _p(k_pages), _p(v_pages), _p(block_table), block_table.shape[1], _p(row_seg),
-        _p(row_pos), rows, num_heads, num_kv_heads, head_dim, ctypes.c_float(scale), int(window), PAGE_SIZE, pages,
+        _p(row_pos), rows, num_heads, num_kv_heads, head_dim, v_dim, ctypes.c_float(scale), int(window), PAGE_SIZE, pages,
         _stream()))
     return out
 
@@ -977,14 +984,15 @@ def attention_is_tiled(head_dim: int) -> bool:
 def attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, k_pages: torch.Tensor,
               v_pages: torch.Tensor, block_table: torch.Tensor, ctx, scale: float, window: int = 0,
               tile_seg: Optional[torch.Tensor] = None, tile_row0: Optional[torch.Tensor] = None,
-              decode_work: Optional[torch.Tensor] = None) -> torch.Tensor:
+              decode_work: Optional[torch.Tensor] = None, v_dim: Optional[int] = None) -> torch.Tensor:
     """bfloat16 with a head size in steps of 16 runs on the matrix cores: the split-key decode
     kernel for segments of one row (all of them, or those a mixed step begins with: a single row
     would hold a 64-row tile of the prompt kernel and walk its whole context alone), the tiled
     kernel for the rest (``tile_seg``, ``tile_row0``: the tiles of ``query_tiles`` in the order
     workgroups take them, those of the leading single rows in front; ``decode_work``: see
-    ``attention_decode``); float32 and everything else on the generic kernel."""
-    fast = q.dtype == torch.bfloat16 and attention_is_tiled(head_dim)
+    ``attention_decode``); float32, value heads of another size than the keys' (``v_dim``) and
+    everything else on the generic kernel."""
+    fast = q.dtype == torch.bfloat16 and attention_is_tiled(head_dim) and v_dim in (None, head_dim)
     if fast and ctx.all_decode:
         return attention_decode(q, num_heads, num_kv_heads, head_dim, k_pages, v_pages, block_table, ctx.row_seg,
                                 ctx.row_pos, scale, ctx.max_context, window, decode_work=decode_work)
@@ -1008,4 +1016,127 @@ def attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
                                  tile_seg[single:], tile_row0[single:], ctx.seg_row0, ctx.row_pos, scale, window,
                                  heads_together=together, out=out)
     return attention_generic(q, num_heads, num_kv_heads, head_dim, k_pages, v_pages, block_table, ctx.row_seg,
-                             ctx.row_pos, scale, window)
+                             ctx.row_pos, scale, window, v_dim=v_dim)
+
+
+# ---- the gated delta rule -----------------------------------------------------------------------------
+def delta_prepare(proj: torch.Tensor, beta_col: int, a: torch.Tensor, taps: torch.Tensor, conv_state: torch.Tensor,
+                  A_log: torch.Tensor, dt_bias: torch.Tensor, row_seg: torch.Tensor, seg_row0: torch.Tensor,
+                  seg_slot: torch.Tensor, segments: int, heads: int, kv_heads: int, dim: int, vdim: int):
+    """From a step's projections to what the recurrence reads. ``proj`` [rows, >= channels + ...]:
+    its first ``channels`` = 2 kv_heads dim + heads vdim columns are q | k | v before their short
+    convolutions, columns ``beta_col`` .. + heads the write strengths before the sigmoid; ``a``
+    [rows, heads dim] the decays' arguments. ``conv_state`` [slots, channels, taps - 1] is read and
+    moved on. Returns float32 (qkv [rows, channels], decay [rows, heads dim], beta [rows, heads])."""
+    _dev(proj, a, taps, conv_state, A_log, dt_bias, row_seg, seg_row0, seg_slot)
+    rows, stride = proj.shape
+    channels = 2 * kv_heads * dim + heads * vdim
+    count = taps.shape[1]
+    if proj.dtype != a.dtype or not proj.is_contiguous() or not a.is_contiguous():
+        raise KernelError("delta_prepare: the projections and the decays' arguments come in one dtype, contiguous")
+    if a.shape != (rows, heads * dim):
+        raise KernelError(f"delta_prepare: a is {tuple(a.shape)}, expected {(rows, heads * dim)}")
+    for name, t, shape in (("taps", taps, (channels, count)), ("A_log", A_log, (heads,)), ("dt_bias", dt_bias, (heads * dim,))):
+        _want(t, torch.float32, name)
+        if t.shape != shape or not t.is_contiguous():
+            raise KernelError(f"delta_prepare: {name} is {tuple(t.shape)}, expected {shape}")
+    _want(conv_state, torch.float32, "conv_state")
+    if conv_state.dim() != 3 or conv_state.shape[1:] != (channels, count - 1) or not conv_state.is_contiguous():
+        raise KernelError(f"delta_prepare: the convolutions' state is {tuple(conv_state.shape)}, expected [slots, {channels}, {count - 1}]")
+    for name, t, n in (("row_seg", row_seg, rows), ("seg_row0", seg_row0, segments + 1), ("seg_slot", seg_slot, segments)):
+        _want(t, torch.int32, name)
+        if t.numel() < n:
+            raise KernelError(f"delta_prepare: {name} holds {t.numel()} entries, needs {n}")
+    qkv = torch.empty((rows, channels), dtype=torch.float32, device=proj.device)
+    decay = torch.empty((rows, heads * dim), dtype=torch.float32, device=proj.device)
+    beta = torch.empty((rows, heads), dtype=torch.float32, device=proj.device)
+    _check(library().fw_delta_prepare(_p(proj), _code(proj.dtype), stride, int(beta_col), _p(a), _p(taps), _p(conv_state), _p(A_log),
+                                      _p(dt_bias), _p(row_seg), _p(seg_row0), _p(seg_slot), _p(qkv), _p(decay), _p(beta), rows,
+                                      int(segments), heads, kv_heads, dim, vdim, count, conv_state.shape[0], _stream()))
+    return qkv, decay, beta
+
+
+def gated_delta_rule(qkv: torch.Tensor, decay: torch.Tensor, beta: torch.Tensor, state: torch.Tensor, seg_row0: torch.Tensor,
+                     seg_slot: torch.Tensor, segments: int, heads: int, kv_heads: int, dim: int, vdim: int) -> torch.Tensor:
+    """The recurrence over each segment's rows; ``state`` [slots, heads, vdim, dim] float32 (the
+    matrix transposed) is read at a segment's start and written at its end. Returns [rows, heads vdim]."""
+    _dev(qkv, decay, beta, state, seg_row0, seg_slot)
+    rows = qkv.shape[0]
+    for name, t, shape in (("qkv", qkv, (rows, 2 * kv_heads * dim + heads * vdim)), ("decay", decay, (rows, heads * dim)),
+                           ("beta", beta, (rows, heads))):
+        _want(t, torch.float32, name)
+        if t.shape != shape or not t.is_contiguous():
+            raise KernelError(f"gated_delta_rule: {name} is {tuple(t.shape)}, expected {shape}")
+    _want(state, torch.float32, "state")
+    if state.dim() != 4 or state.shape[1:] != (heads, vdim, dim) or not state.is_contiguous():
+        raise KernelError(f"gated_delta_rule: the state is {tuple(state.shape)}, expected [slots, {heads}, {vdim}, {dim}]")
+    for name, t, n in (("seg_row0", seg_row0, segments + 1), ("seg_slot", seg_slot, segments)):
+        _want(t, torch.int32, name)
+        if t.numel() < n:
+            raise KernelError(f"gated_delta_rule: {name} holds {t.numel()} entries, needs {n}")
+    out = torch.empty((rows, heads * vdim), dtype=torch.float32, device=qkv.device)
+    _check(library().fw_gated_delta_rule(_p(qkv), _p(decay), _p(beta), _p(state), _p(out), _p(seg_row0), _p(seg_slot), rows,
+                                         int(segments), heads, kv_heads, dim, vdim, state.shape[0], _stream()))
+    return out
+
+
+def gated_head_norm(o: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, heads: int, vdim: int, eps: float,
+                    out_dtype: torch.dtype) -> torch.Tensor:
+    """Per head: o / rms(o) * weight * sigmoid(gate); ``o`` float32 [rows, heads vdim], ``gate``
+    [rows, heads vdim] (float32, or bfloat16 beside a bfloat16 output)."""
+    _dev(o, gate, weight)
+    _want(o, torch.float32, "o")
+    _want(weight, torch.float32, "weight")
+    rows = o.shape[0]
+    if o.shape != (rows, heads * vdim) or gate.shape != o.shape or weight.shape != (vdim,) or not o.is_contiguous() or not gate.is_contiguous():
+        raise KernelError(f"gated_head_norm: o {tuple(o.shape)}, gate {tuple(gate.shape)}, weight {tuple(weight.shape)} do not fit {heads} x {vdim}")
+    out = torch.empty((rows, heads * vdim), dtype=out_dtype, device=o.device)
+    _check(library().fw_gated_head_norm(_p(o), _p(gate), _code(gate.dtype), heads * vdim, _p(weight), _p(out), _code(out_dtype), rows,
+                                        heads, vdim, ctypes.c_float(eps), _stream()))
+    return out
+
+
+# ---- sublayers whose output is normed --------------------------------------------------------------------
+def norm_scale_add_(x: torch.Tensor, a: torch.Tensor, weight: torch.Tensor, eps: float, mult: float, *,
+                    b: Optional[torch.Tensor] = None, scale_a: float = 1.0, scale_b: float = 1.0,
+                    one_centered: bool = False, rounded_dtype: Optional[torch.dtype] = None) -> Optional[torch.Tensor]:
+    """x += mult * rmsnorm(scale_a a + scale_b b) * w in place (float32 rows; ``b`` optional). With
+    ``rounded_dtype`` the new x is also returned in that dtype (what the next products read)."""
+    _dev(x, a, b, weight)
+    rows, hidden = x.shape
+    for name, t in (("x", x), ("a", a), ("b", b)):
+        if t is not None:
+            _want(t, torch.float32, name)
+            if t.shape != (rows, hidden) or not t.is_contiguous():
+                raise KernelError(f"norm_scale_add: {name} is {tuple(t.shape)}, expected {(rows, hidden)}")
+    _want(weight, torch.float32, "weight")
+    if weight.shape != (hidden,):
+        raise KernelError(f"norm_scale_add: weight is {tuple(weight.shape)}, row width is {hidden}")
+    rounded = torch.empty((rows, hidden), dtype=rounded_dtype, device=x.device) if rounded_dtype is not None else None
+    _check(library().fw_norm_scale_add(_p(x), _p(a), _p(b), ctypes.c_float(scale_a), ctypes.c_float(scale_b), _p(weight),
+                                       int(one_centered), ctypes.c_float(eps), ctypes.c_float(mult), _p(rounded),
+                                       _code(rounded_dtype) if rounded_dtype is not None else F32, rows, hidden, _stream()))
+    return rounded
+
+
+def round_rows(x: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    """float32 rows in the activation dtype (float32: the rows themselves)."""
+    _want(x, torch.float32, "x")
+    if dtype == torch.float32:
+        return x
+    _dev(x)
+    out = torch.empty(x.shape, dtype=torch.bfloat16, device=x.device)
+    _check(library().fw_round_rows(_p(x), _p(out), ctypes.c_longlong(x.numel()), _stream()))
+    return out
+
+
+def clamped_glu(gate_up: torch.Tensor, limit: float, alpha: float, shift: float, out_dtype: torch.dtype) -> torch.Tensor:
+    """[rows, gate | up] -> min(gate, limit) * sigmoid(alpha * that) * (clamp(up, +-limit) + shift)."""
+    _dev(gate_up)
+    rows, width = gate_up.shape
+    if width % 2 or not gate_up.is_contiguous():
+        raise KernelError("clamped_glu: the input holds gate and up halves, contiguous")
+    out = torch.empty((rows, width // 2), dtype=out_dtype, device=gate_up.device)
+    _check(library().fw_clamped_glu(_p(gate_up), _code(gate_up.dtype), _p(out), _code(out_dtype), rows, width // 2,
+                                    ctypes.c_float(limit), ctypes.c_float(alpha), ctypes.c_float(shift), _stream()))
+    return out

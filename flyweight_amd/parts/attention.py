@@ -2,8 +2,10 @@
 
 q = W_q h, k = W_k h, v = W_v h; optional per-head RMS norm of q and k (one weight of
 head_dim shared by all heads); position encoding on q and k; k and v appended to the
-cache; scores q.k / sqrt(head_dim) over the cached keys the row may see (causal, optionally
-only the last ``window``), softmax in float32, weighted sum of values; out = W_o o.
+cache; scores q.k * softmax_scale (1 / sqrt(head_dim) unless given) over the cached keys the row
+may see (causal, optionally only the last ``window``: itself and the window - 1 before it),
+softmax in float32, weighted sum of values; out = W_o o. Values may have a size of their own
+(``v_head_dim``); the output of a head has that size.
 Query head i reads kv head i // (num_heads / num_kv_heads). Formulas as the reference's
 LFM2 attention branch computes them (native/src/v2_runtime.cpp:28429-28478).
 """
@@ -40,24 +42,32 @@ class GQAttention(Mixer):
         self.num_heads = int(spec["num_heads"])
         self.num_kv_heads = int(spec["num_kv_heads"])
         self.head_dim = int(spec["head_dim"])
+        self.v_head_dim = int(spec.get("v_head_dim") or self.head_dim)
         self.qk_norm = bool(spec.get("qk_norm", False))
         self.qk_norm_eps = float(spec.get("qk_norm_eps", 1e-6)) if self.qk_norm else 1.0
         self.window = spec.get("window")
         self.scale = float(spec.get("softmax_scale", self.head_dim ** -0.5))
         self.bias = bool(spec.get("bias", False))
         self.names = {**_DEFAULT_NAMES, **dict(spec.get("names", {}))}
+        # what follows a tensor's name in the checkpoint: ".weight" / ".bias" unless the layout has none
+        self.weight_suffix = spec.get("weight_suffix", ".weight")
         self.position = build_part("position", spec["position"])
         if self.num_heads % self.num_kv_heads:
             raise ConfigError(f"{self.num_heads} heads are not a multiple of {self.num_kv_heads} kv heads")
-        if self.head_dim > ops.MAX_HEAD_DIM:
-            raise ConfigError(f"head_dim {self.head_dim} exceeds the kernels' limit of {ops.MAX_HEAD_DIM}")
+        if max(self.head_dim, self.v_head_dim) > ops.MAX_HEAD_DIM:
+            raise ConfigError(f"head_dim {self.head_dim} / value size {self.v_head_dim} exceeds the kernels' limit of {ops.MAX_HEAD_DIM}")
+        if self.bias and self.weight_suffix != ".weight":
+            raise ConfigError("biases need the '.weight' / '.bias' tensor names")
         if self.window is not None and int(self.window) <= 0:
             raise ConfigError("an attention window must be positive (or None for all keys)")
 
     def cache_need(self):
-        return PagedKV(self.num_kv_heads, self.head_dim, None if self.window is None else int(self.window))
+        return PagedKV(self.num_kv_heads, self.head_dim, None if self.window is None else int(self.window),
+                       None if self.v_head_dim == self.head_dim else self.v_head_dim)
 
     def _name(self, which: str, leaf: str = "weight") -> str:
+        if leaf == "weight":
+            return f"{self.prefix}{self.names[which]}{self.weight_suffix}"
         return f"{self.prefix}{self.names[which]}.{leaf}"
 
     def tensors(self) -> Dict[str, TensorDecl]:
@@ -65,8 +75,8 @@ class GQAttention(Mixer):
         declared = {
             self._name("q"): TensorDecl((q_width, self.hidden)),
             self._name("k"): TensorDecl((kv_width, self.hidden)),
-            self._name("v"): TensorDecl((kv_width, self.hidden)),
-            self._name("o"): TensorDecl((self.hidden, q_width)),
+            self._name("v"): TensorDecl((self.num_kv_heads * self.v_head_dim, self.hidden)),
+            self._name("o"): TensorDecl((self.hidden, self.num_heads * self.v_head_dim)),
         }
         if self.bias:
             declared[self._name("q", "bias")] = TensorDecl((q_width,), "vector", "bias")
@@ -99,7 +109,8 @@ class GQAttention(Mixer):
     RUN_OF_KEYS = ops.DECODE_SPLIT_PAGES * ops.PAGE_SIZE
 
     def step_arrays_key(self):
-        fast = getattr(self, "dtype", None) == torch.bfloat16 and ops.attention_is_tiled(self.head_dim)
+        fast = getattr(self, "dtype", None) == torch.bfloat16 and ops.attention_is_tiled(self.head_dim) \
+            and self.v_head_dim == self.head_dim
         return ("query_tiles", ops.QUERY_TILE, self.RUN_OF_KEYS) if fast else None
 
     def _decode_work(self, batch) -> int:
@@ -126,23 +137,32 @@ class GQAttention(Mixer):
     def refresh_step_arrays(self, batch, arrays) -> None:
         arrays["decode_work"][0] = self._decode_work(batch)     # the tiles of single rows never change
 
-    def forward(self, h, residual, ctx, cache):
+    def attend(self, h, ctx, cache) -> torch.Tensor:
+        """The heads' outputs [rows, heads * v_head_dim] in the activation dtype, the step's keys and
+        values appended to the cache on the way."""
         qkv = self.qkv.forward(h, out_dtype=torch.float32)      # normed, rotated and rounded once, below
         cos, sin = ctx.position_tables(self.position)
         own = ctx.step_arrays(self) if self.step_arrays_key() is not None else {}
         if ctx.all_decode and ctx.num_rows <= self.FUSED_DECODE_ROWS and qkv.dtype == torch.float32 and self.step_arrays_key() is not None:
             # a few single-token segments on the matrix cores: norm, rotation, cache write and attention in one kernel
-            attended = ops.attention_decode_fused(
+            return ops.attention_decode_fused(
                 qkv, self.num_heads, self.num_kv_heads, self.head_dim, self.q_norm_weight, self.k_norm_weight, self.qk_norm_eps,
                 cos, sin, self.position.rotary_dim, cache.k_pages, cache.v_pages, cache.block_table, ctx.row_seg, ctx.row_pos,
                 self.scale, ctx.max_context, int(self.window or 0), write_kv=cache.writes,
                 decode_work=own.get("decode_work"))
-            return self.out.accumulate(attended, residual, then=getattr(ctx, "upcoming_norm", None))
         q = ops.qk_norm_rope_kv_write(
             qkv, self.num_heads, self.num_kv_heads, self.head_dim, self.q_norm_weight, self.k_norm_weight,
             self.qk_norm_eps, cos, sin, self.position.rotary_dim, cache.k_pages, cache.v_pages, cache.block_table,
-            ctx.row_seg, ctx.row_pos, write_kv=cache.writes)
-        attended = ops.attention(q, self.num_heads, self.num_kv_heads, self.head_dim, cache.k_pages, cache.v_pages,
-                                 cache.block_table, ctx, self.scale, int(self.window or 0),
-                                 tile_seg=own.get("tile_seg"), tile_row0=own.get("tile_row0"), decode_work=own.get("decode_work"))
-        return self.out.accumulate(attended, residual, then=getattr(ctx, "upcoming_norm", None))
+            ctx.row_seg, ctx.row_pos, write_kv=cache.writes, v_dim=self.v_head_dim)
+        return ops.attention(q, self.num_heads, self.num_kv_heads, self.head_dim, cache.k_pages, cache.v_pages,
+                             cache.block_table, ctx, self.scale, int(self.window or 0),
+                             tile_seg=own.get("tile_seg"), tile_row0=own.get("tile_row0"), decode_work=own.get("decode_work"),
+                             v_dim=self.v_head_dim)
+
+    def forward(self, h, residual, ctx, cache):
+        return self.out.accumulate(self.attend(h, ctx, cache), residual, then=getattr(ctx, "upcoming_norm", None))
+
+    def output(self, h, ctx, cache) -> torch.Tensor:
+        """The mixer's output as float32 rows of its own (for arrangements that do something to it
+        before it joins the residual stream)."""
+        return self.out.forward(self.attend(h, ctx, cache), out_dtype=torch.float32)

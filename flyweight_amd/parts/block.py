@@ -3,10 +3,16 @@
 ``pre_norm_residual``: x <- x + mixer(norm1(x)); x <- x + ffn(norm2(x)), the residual
 stream x in float32 (native/src/v2_runtime.cpp:28077,28282,28774,29133-29136). Another
 arrangement (post-norm, parallel mixer and feed-forward) is another class registered here.
+
+``output_norm_residual``: x <- x + m * norm1(mixer(x)); x <- x + m * norm2(ffn(x)). The sublayers
+read x itself (rounded to the activation dtype for their products), the norm stands on a
+sublayer's OUTPUT, and m is a fixed factor. The feed-forward may be absent.
 """
 
 from __future__ import annotations
 
+from ..config.spec import ConfigError
+from ..kernels import ops
 from .base import Block, build_part, register_block
 from .norm import LazyNorm
 
@@ -47,3 +53,72 @@ class PreNormResidualBlock(Block):
         prepared = self.ffn.forward(h if getattr(self.ffn, "accepts_lazy_norm", False) else h.tensor(), x, ctx)
         ctx.upcoming_norm = None
         return prepared
+
+
+class RoundedRows:
+    """The residual rows once more in the activation dtype, left by the kernel that last changed
+    them, for the block that reads them next. (``norm`` is None: a block that looks for a prepared
+    norm finds none here.)"""
+    norm = None
+
+    def __init__(self, activations):
+        self.activations = activations
+
+
+@register_block("output_norm_residual")
+class OutputNormResidualBlock(Block):
+    def __init__(self, spec):
+        self.spec = spec
+        self.mixer_norm = build_part("norm", spec.mixer_norm)
+        self.mixer = build_part("mixer", spec.mixer)
+        self.ffn = build_part("ffn", spec.ffn) if spec.ffn is not None else None
+        self.ffn_norm = build_part("norm", spec.ffn_norm) if spec.ffn is not None else None
+        self.mult = float(spec.params.get("residual_mult", 1.0))
+        for norm in (self.mixer_norm, self.ffn_norm):
+            if norm is not None and not hasattr(norm, "rms_parameters"):
+                raise ConfigError("the output-norm arrangement takes RMS norms")
+
+    def parts(self):
+        return tuple(part for part in (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn) if part is not None)
+
+    def cache_need(self):
+        return self.mixer.cache_need()
+
+    @property
+    def graph_safe(self) -> bool:
+        position = getattr(self.mixer, "position", None)
+        return all(part.graph_safe for part in self.parts()) and (position is None or position.graph_safe)
+
+    def _terms(self, part, *args):
+        """A sublayer's output as [(float32 rows, scale)]: from the part itself if it can say so,
+        else by letting it add into rows of zeros."""
+        if hasattr(part, "output_terms"):
+            return part.output_terms(*args)
+        if hasattr(part, "output"):
+            return [(part.output(*args), 1.0)]
+        raise ConfigError(f"part '{part.spec.kind}' cannot give its output apart from the residual stream")
+
+    def _join(self, x, terms, norm, dtype):
+        """x += m * norm(sum of the terms); returns the new x rounded for the next reader."""
+        weight, eps, one_centered = norm.rms_parameters()
+        while len(terms) > 2:       # more than two branches: the last two are summed first
+            (a, sa), (b, sb) = terms[-2], terms[-1]
+            a = a * sa
+            a.add_(b, alpha=sb)
+            terms = terms[:-2] + [(a, 1.0)]
+        (a, scale_a), (b, scale_b) = terms[0], terms[1] if len(terms) > 1 else (None, 1.0)
+        return ops.norm_scale_add_(x, a, weight, eps, self.mult, b=b, scale_a=scale_a, scale_b=scale_b,
+                                   one_centered=one_centered, rounded_dtype=None if dtype == x.dtype else dtype)
+
+    def forward(self, x, ctx, cache, prepared=None, norm_after=None):
+        """``x`` [rows, hidden] float32 is updated in place."""
+        dtype = self.mixer_norm.dtype
+        if isinstance(prepared, RoundedRows) and prepared.activations.shape == x.shape and prepared.activations.dtype == dtype:
+            h = prepared.activations
+        else:
+            h = ops.round_rows(x, dtype)
+        rounded = self._join(x, self._terms(self.mixer, h, ctx, cache), self.mixer_norm, dtype)
+        if self.ffn is not None:
+            h = x if rounded is None else rounded
+            rounded = self._join(x, self._terms(self.ffn, h, ctx), self.ffn_norm, dtype)
+        return None if rounded is None else RoundedRows(rounded)

@@ -64,12 +64,18 @@ class RMSNorm(Norm):
         self.eps = float(spec["eps"])
         self.one_centered = bool(spec.get("one_centered", False))
 
+    @property
+    def tensor_name(self) -> str:
+        """``prefix`` + "weight", unless the layout names the tensor itself (``tensor``)."""
+        return self.spec.get("tensor") or self.prefix + "weight"
+
     def tensors(self) -> Dict[str, TensorDecl]:
-        return {self.prefix + "weight": TensorDecl((self.size,), role="vector", init="norm")}
+        # a weight stored around zero (used as 1 + w) starts around zero
+        return {self.tensor_name: TensorDecl((self.size,), role="vector", init="bias" if self.one_centered else "norm")}
 
     def bind(self, tensors, dtype, device) -> None:
         super().bind(tensors, dtype, device)
-        self.weight = tensors[self.prefix + "weight"]
+        self.weight = tensors[self.tensor_name]
 
     def rms_parameters(self):
         return self.weight, self.eps, self.one_centered

@@ -2,7 +2,8 @@
 i + rotary_dim/2, angle = position * theta^(-2i/rotary_dim); channels past ``rotary_dim``
 pass through (native/include/flyweight_v2_native_kernels.hpp:993-1050). The inverse
 frequencies are formed in float64 on the host; the per-step cos/sin tables are float32.
-``rotary_dim = 0`` (or kind ``none``) means no position encoding at all."""
+``rotary_dim = 0`` (or kind ``none``) means no position encoding at all. ``scaling_factor`` f
+(linear position scaling) divides every frequency by f: position p turns as p / f would."""
 
 from __future__ import annotations
 
@@ -22,6 +23,9 @@ class RotaryNeox(PositionEncoding):
         self.theta = float(spec["theta"])
         self.head_dim = int(spec["head_dim"])
         self.rotary_dim = int(spec.get("rotary_dim", self.head_dim))
+        self.scaling_factor = float(spec.get("scaling_factor", 1.0))
+        if not self.scaling_factor > 0.0:
+            raise ConfigError(f"the rotation's scaling factor must be positive, found {self.scaling_factor}")
         if self.rotary_dim % 2 or not 0 <= self.rotary_dim <= self.head_dim:
             raise ConfigError(f"rotary_dim {self.rotary_dim} must be even and at most head_dim {self.head_dim}")
         self._inv_freq = None
@@ -30,7 +34,7 @@ class RotaryNeox(PositionEncoding):
         super().bind(tensors, dtype, device)
         half = self.rotary_dim // 2
         exponents = torch.arange(half, dtype=torch.float64) * 2.0 / max(self.rotary_dim, 1)
-        self._inv_freq = (self.theta ** (-exponents)).to(device)
+        self._inv_freq = (self.theta ** (-exponents) / self.scaling_factor).to(device)
 
     def tables(self, ctx):
         if self.rotary_dim == 0:
