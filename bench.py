@@ -51,6 +51,101 @@ WORKLOADS = {
 }
 
 
+# Koketar (windowed attention beside a gated delta rule in every layer) at sizes that resemble a real model's
+# layers, each beside the engine's closest existing model, an LFM2 of the same width, depth, feed-forward
+# width and vocabulary (half its layers attention over every key, half gated short convolutions).
+KOKETAR_SIZES = {
+    "w1024": dict(width=1024, layers=4, vocab=32768, ff=4096, heads=8, kv_heads=2, dim=128, vdim=128, window=512, rot_dims=64,
+                  r_heads=8, r_kv_heads=4, r_dim=64, r_vdim=128, conv=4, rank=32),
+    "w2048": dict(width=2048, layers=4, vocab=32768, ff=8192, heads=16, kv_heads=4, dim=128, vdim=128, window=1024, rot_dims=64,
+                  r_heads=16, r_kv_heads=8, r_dim=128, r_vdim=128, conv=4, rank=64),
+}
+
+
+def koketar_configs(size: dict):
+    """(Koketar configuration, LFM2 configuration of equal size)."""
+    from flyweight_amd.config import config_from_dict
+    layer = {"type": "parallel", "mlp": {"kind": "dense", "ff": size["ff"], "limit": 7.0},
+             "mixer": {"left_scale": 1.0, "right_scale": 1.0,
+                       "left": {"heads": size["heads"], "kv_heads": size["kv_heads"], "dim": size["dim"], "vdim": size["vdim"],
+                                "scale": size["dim"] ** -0.5, "mask": {"size": size["window"]},
+                                "rot": {"dims": size["rot_dims"], "base": 1000000.0, "scaling": {"factor": 4.0}}},
+                       "right": {"heads": size["r_heads"], "kv_heads": size["r_kv_heads"], "dim": size["r_dim"], "vdim": size["r_vdim"],
+                                 "conv": size["conv"], "decay_rank": size["rank"], "gate_rank": size["rank"]}}}
+    koketar = config_from_dict({"architecture": "Koketar", "vocab": size["vocab"], "width": size["width"], "norm": {"eps": 1e-5},
+                                "residual_mult": 0.5, "logit_softcap": 30.0, "layers": [layer] * size["layers"]})
+    lfm2 = config_from_dict(dict(
+        architectures=["Lfm2ForCausalLM"], model_type="lfm2", vocab_size=size["vocab"], hidden_size=size["width"],
+        num_hidden_layers=size["layers"], num_attention_heads=size["width"] // 64, num_key_value_heads=size["width"] // 256,
+        intermediate_size=size["ff"], block_auto_adjust_ff_dim=False, norm_eps=1e-5, rope_theta=1000000.0, conv_L_cache=3,
+        conv_bias=False, tie_word_embeddings=True, max_position_embeddings=CONTEXT,
+        layer_types=["conv", "full_attention"] * (size["layers"] // 2)))
+    return koketar, lfm2
+
+
+def kernel_times(torch, run) -> dict:
+    """Entry point of the kernel library -> microseconds of GPU time per call, over one call of ``run``
+    (launched kernel by kernel, every call bracketed by two events)."""
+    from flyweight_amd.kernels import ops
+    ops.kernel_profile(True)
+    try:
+        run()
+        report = ops.kernel_profile_report()
+    finally:
+        ops.kernel_profile(False)
+    return {name: {"calls": int(t["calls"]), "us_per_call": round(t["gpu_ms"] * 1e3 / max(t["calls"], 1), 2),
+                   "us": round(t["gpu_ms"] * 1e3, 1)} for name, t in report.items()}
+
+
+def koketar_run(torch, args) -> dict:
+    """Prefill (one step of 2,048 prompt tokens) and decode (batch 8 and 64 behind 2,048-token prompts) of
+    Koketar and of the LFM2 of equal size, tokens a second, with the time of every kernel of a prompt's step
+    and of a decode step at batch 8."""
+    from flyweight_amd import Model, Runtime, StepEntry
+    import numpy as np
+    results = {}
+    steps = min(args.steps, 64)
+    for size_name, size in KOKETAR_SIZES.items():
+        for family, config in zip(("koketar", "lfm2"), koketar_configs(size)):
+            log(f"{family} {size_name}: random bfloat16 weights")
+            model = Model.random(config, seed=0, dtype="bfloat16")
+            record = {}
+            seconds, flops = prefill_run(torch, model, config, repeats=3)
+            record["prefill_2048_tokens_per_s"] = round(PROMPT / seconds, 1)
+            record["prefill_2048_ms"] = round(seconds * 1e3, 3)
+            record["prefill_2048_frac_of_bf16_peak"] = round(flops / seconds / MFMA_BF16_PEAK, 4)
+            for batch in (8, 64):
+                seconds, _, step_bytes = decode_run(torch, model, config, batch, steps, min(args.warmup, 8))
+                record[f"decode_b{batch}_tokens_per_s"] = round(batch * steps / seconds, 1)
+                record[f"decode_b{batch}_ms_per_step"] = round(seconds / steps * 1e3, 4)
+                record[f"decode_b{batch}_frac_of_hbm_peak"] = round(step_bytes / (seconds / steps) / 1e9 / HBM_PEAK_GBS, 4)
+            # kernel by kernel: a prompt's step, and a decode step of 8 requests behind their prompts
+            rng = np.random.default_rng(4)
+            runtime = Runtime(model, context_limit=CONTEXT, parallel_sequences=8, num_pages=8 * (PROMPT // 64 + 1)).prepare()
+            for request in range(8):
+                runtime.admit(request)
+            prompts = [rng.integers(0, config.vocab_size, PROMPT).tolist() for _ in range(8)]
+            runtime.step([StepEntry(0, prompts[0], [PROMPT - 1])])
+            record["kernels_prefill_2048"] = kernel_times(torch, lambda: runtime.step([StepEntry(1, prompts[1], [PROMPT - 1])]))
+            for request in range(2, 8):
+                runtime.step([StepEntry(request, prompts[request], [])])
+            one_each = lambda: runtime.step([StepEntry(request, [1], [0]) for request in range(8)])
+            one_each()
+            record["kernels_decode_b8"] = kernel_times(torch, one_each)
+            runtime.close()
+            results[f"{family}_{size_name}"] = record
+            del model, runtime
+            torch.cuda.empty_cache()
+    headline = results["koketar_w2048"]
+    return {"metric": "decode tok/s @ batch 8 (Koketar, width 2,048, 4 layers, 2,048-token prompts)",
+            "value": headline["decode_b8_tokens_per_s"], "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": min(args.warmup, 8),
+            "ms_per_step": headline["decode_b8_ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "bf16", "data": "synthetic: seeded uniform token ids, random-init weights",
+            "config": {"model": "Koketar beside LFM2 at equal width, depth, feed-forward width and vocabulary", "sizes": KOKETAR_SIZES,
+                       "prompt_len": PROMPT, "seq_len": CONTEXT, "parallelism": "single GPU"},
+            "results": results}
+
+
 def log(text: str) -> None:
     print(f"[bench] {text}", file=sys.stderr, flush=True)
 
@@ -347,8 +442,9 @@ def main() -> int:
     parser.add_argument("--only", choices=("decode", "prefill"), help="run one phase and print no JSON (for profiling)")
     parser.add_argument("--drawn", action="store_true", help="with --only decode: the requests draw their tokens "
                         "(temperature 0.8, top_k 40, top_p 0.95, min_p 0.05) instead of taking the most likely one")
-    parser.add_argument("--workload", choices=("headline",) + tuple(WORKLOADS), default="headline",
-                        help="headline: the LFM2-1.2B decode and prefill figures; the others: a whole serving run")
+    parser.add_argument("--workload", choices=("headline",) + tuple(WORKLOADS) + ("koketar",), default="headline",
+                        help="headline: the LFM2-1.2B decode and prefill figures; long-context, mixed: a whole serving run; "
+                             "koketar: prefill and decode of Koketar beside LFM2 at equal sizes, kernel by kernel")
     parser.add_argument("--requests", type=int, help="requests of a serving workload (default: as the workload names)")
     args = parser.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -362,6 +458,9 @@ def main() -> int:
     from flyweight_amd import Model
     from flyweight_amd.config import config_from_dict
 
+    if args.workload == "koketar":
+        print(json.dumps(koketar_run(torch, args)), flush=True)
+        return 0
     if args.workload != "headline":
         print(json.dumps(serving_run(torch, args.workload, args.requests or WORKLOADS[args.workload]["requests"])), flush=True)
         return 0

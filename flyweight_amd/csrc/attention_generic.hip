@@ -275,10 +275,10 @@ extern "C" int fw_attention_generic(const void* q, void* out, int dtype, const v
                                     const int32_t* row_seg, const int32_t* row_pos, int rows, int num_heads,
                                     int num_kv_heads, int head_dim, int v_dim, float scale, int window, int page_size,
                                     int num_pages, void* stream) {
-    FW_REQUIRE(v_dim > 0 && v_dim <= ATTN_MAX_HEAD_DIM, "attention: value size %d outside 1..%d", v_dim, ATTN_MAX_HEAD_DIM);
     FW_REQUIRE(rows >= 0 && num_heads > 0 && num_kv_heads > 0 && num_heads % num_kv_heads == 0,
                "attention: heads %d must be a positive multiple of kv heads %d", num_heads, num_kv_heads);
     FW_REQUIRE(head_dim > 0 && head_dim <= ATTN_MAX_HEAD_DIM, "attention: head_dim %d outside 1..%d", head_dim, ATTN_MAX_HEAD_DIM);
+    FW_REQUIRE(v_dim > 0 && v_dim <= ATTN_MAX_HEAD_DIM, "attention: value size %d outside 1..%d", v_dim, ATTN_MAX_HEAD_DIM);
     FW_REQUIRE(page_size == ATTN_PAGE, "attention: page size must be %d, got %d", ATTN_PAGE, page_size);
     FW_REQUIRE(window >= 0, "attention: window must be 0 (all keys) or positive, got %d", window);
     FW_REQUIRE(num_pages > 0 && table_stride > 0, "attention: empty cache (pages=%d, table stride=%d)", num_pages, table_stride);

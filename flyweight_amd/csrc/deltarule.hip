@@ -6,8 +6,10 @@
 //     S <- diag(g) S;   u = beta (v - S^T k);   S <- S + k u^T;   o = S^T q
 // so the read-out sees the token's own write. Columns of S (value channels) never meet: a column is
 // owned by four lanes, each holding a quarter of its rows in registers, and the two sums over the
-// key channels are reductions over those four lanes. A segment's tokens are walked in order; what a
-// token brings is staged through LDS a chunk of tokens at a time.
+// key channels are reductions over those four lanes. A segment's tokens are walked in order. What a
+// token brings to a head lies in one record, [q | k | g | beta | v] (fw_delta_record_floats), so that a
+// chunk of tokens is a plain copy into LDS; the copy of the next chunk is asked for before the work on
+// this one and waits in registers meanwhile.
 //
 // The state is stored transposed, [slot][head][vdim][dim], so that the quarter columns a wave holds
 // are one contiguous piece of memory.
@@ -27,24 +29,29 @@ __device__ __forceinline__ float fw_softplus(float x) { return x > 20.0f ? x : l
 // g = exp(-exp(A_log[h]) * softplus(a + dt_bias)); lane 0 of a decay vector also forms beta.
 // proj [rows][proj_stride]: columns 0.. hold q | k | v (the convolution's inputs), column beta_col + h
 // the write strength before its sigmoid. state [slots][C][L-1]: the inputs of the L-1 tokens before
-// the segment, oldest first. The state is read here and moved on by conv_state_kernel afterwards.
-template <typename TI>
+// the segment, oldest first. The state is read here and moved on by conv_state_kernel afterwards;
+// with SINGLE (every segment is one row: a decode step) the wave that read a channel's memory moves it
+// on itself. a [rows][a_stride]: the decays' arguments in its first heads * dim columns.
+template <typename TI, bool SINGLE>
 __global__ __launch_bounds__(64) void delta_prepare_kernel(
-    const TI* __restrict__ proj, int proj_stride, int beta_col, const TI* __restrict__ a, const float* __restrict__ taps,
-    const float* __restrict__ conv_state, const float* __restrict__ A_log, const float* __restrict__ dt_bias,
+    const TI* __restrict__ proj, int proj_stride, int beta_col, const TI* __restrict__ a, int a_stride, const float* __restrict__ taps,
+    float* __restrict__ conv_state, const float* __restrict__ A_log, const float* __restrict__ dt_bias,
     const int32_t* __restrict__ row_seg, const int32_t* __restrict__ seg_row0, const int32_t* __restrict__ seg_slot,
-    float* __restrict__ qkv_out, float* __restrict__ decay_out, float* __restrict__ beta_out, int heads, int kv_heads,
-    int dim, int vdim, int taps_count) {
+    float* __restrict__ records, int heads, int kv_heads, int dim, int vdim, int taps_count) {
     const int row = blockIdx.x, vec = blockIdx.y, lane = threadIdx.x;
     const int conv_channels = 2 * kv_heads * dim + heads * vdim;
+    const int d4 = (dim + 3) & ~3, v4 = (vdim + 3) & ~3;
+    const int record = 3 * d4 + 4 + v4;                     // q | k | g | beta and three unused | v
+    float* of_row = records + (size_t)row * heads * record;
     if (vec >= 2 * kv_heads + heads) {      // a decay vector
         const int h = vec - 2 * kv_heads - heads;
         const float rate = expf(A_log[h]);
-        for (int i = lane; i < dim; i += 64) {
+        float* dest = of_row + (size_t)h * record + 2 * d4;
+        for (int i = lane; i < d4; i += 64) {
             const int at = h * dim + i;
-            decay_out[(size_t)row * heads * dim + at] = expf(-rate * fw_softplus(load_as_float(a, (size_t)row * heads * dim + at) + dt_bias[at]));
+            dest[i] = i < dim ? expf(-rate * fw_softplus(load_as_float(a, (size_t)row * a_stride + at) + dt_bias[at])) : 0.0f;
         }
-        if (lane == 0) beta_out[(size_t)row * heads + h] = fw_sigmoid(load_as_float(proj, (size_t)row * proj_stride + beta_col + h));
+        if (lane < 4) dest[d4 + lane] = lane == 0 ? fw_sigmoid(load_as_float(proj, (size_t)row * proj_stride + beta_col + h)) : 0.0f;
         return;
     }
     const bool value = vec >= 2 * kv_heads;
@@ -52,7 +59,7 @@ __global__ __launch_bounds__(64) void delta_prepare_kernel(
     const int c0 = value ? 2 * kv_heads * dim + (vec - 2 * kv_heads) * vdim : vec * dim;
     const int seg = row_seg[row];
     const int first = seg_row0[seg];
-    const float* before = conv_state + (size_t)seg_slot[seg] * conv_channels * (taps_count - 1);
+    float* before = conv_state + (size_t)seg_slot[seg] * conv_channels * (taps_count - 1);
     float sum_sq = 0.0f;
     // a vector of up to 256 channels: four per lane
     float kept[4];
@@ -69,6 +76,8 @@ __global__ __launch_bounds__(64) void delta_prepare_kernel(
                 const float x = r >= first ? load_as_float(proj, (size_t)r * proj_stride + c)
                                            : before[(size_t)c * (taps_count - 1) + (taps_count - 1 + (r - first))];
                 acc = fmaf(taps[(size_t)c * taps_count + j], x, acc);
+                // the memory moves on by this row: entry j - 1 takes x, and no later tap reads it
+                if (SINGLE && j > 0) before[(size_t)c * (taps_count - 1) + j - 1] = x;
             }
             y = acc * fw_sigmoid(acc);
         }
@@ -81,10 +90,19 @@ __global__ __launch_bounds__(64) void delta_prepare_kernel(
         factor = 1.0f / sqrtf(sum_sq + 1e-6f);
         if (vec < kv_heads) factor *= 1.0f / sqrtf((float)dim);
     }
+    // a value head goes to its head's record; a query or key head to the records of every head of its group
+    const int group = heads / kv_heads;
+    const int first_head = value ? vec - 2 * kv_heads : (vec % kv_heads) * group;
+    const int copies = value ? 1 : group;
+    const int at = value ? 3 * d4 + 4 : (vec < kv_heads ? 0 : d4);
+    const int padded = value ? v4 : d4;
+    for (int copy = 0; copy < copies; ++copy) {
+        float* dest = of_row + (size_t)(first_head + copy) * record + at;
 #pragma unroll
-    for (int part = 0; part < 4; ++part) {
-        const int i = lane + 64 * part;
-        if (i < width) qkv_out[(size_t)row * conv_channels + c0 + i] = kept[part] * factor;
+        for (int part = 0; part < 4; ++part) {
+            const int i = lane + 64 * part;
+            if (i < padded) dest[i] = i < width ? kept[part] * factor : 0.0f;
+        }
     }
 }
 
@@ -108,11 +126,10 @@ __global__ void conv_state_kernel(const TI* __restrict__ proj, int proj_stride, 
     }
 }
 
-extern "C" int fw_delta_prepare(const void* proj, int dtype, int proj_stride, int beta_col, const void* a, const float* taps,
+extern "C" int fw_delta_prepare(const void* proj, int dtype, int proj_stride, int beta_col, const void* a, int a_stride, const float* taps,
                                 float* conv_state, const float* A_log, const float* dt_bias, const int32_t* row_seg,
-                                const int32_t* seg_row0, const int32_t* seg_slot, float* qkv_out, float* decay_out,
-                                float* beta_out, int rows, int segments, int heads, int kv_heads, int dim, int vdim,
-                                int taps_count, int slots, void* stream) {
+                                const int32_t* seg_row0, const int32_t* seg_slot, float* records, int rows, int segments,
+                                int heads, int kv_heads, int dim, int vdim, int taps_count, int slots, void* stream) {
     FW_REQUIRE(rows >= 0 && segments >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0,
                "delta_prepare: heads %d must be a positive multiple of kv heads %d", heads, kv_heads);
     FW_REQUIRE(dim > 0 && dim <= 256 && vdim > 0 && vdim <= 256, "delta_prepare: dim %d and vdim %d must lie in 1..256", dim, vdim);
@@ -121,49 +138,100 @@ extern "C" int fw_delta_prepare(const void* proj, int dtype, int proj_stride, in
     const int channels = 2 * kv_heads * dim + heads * vdim;
     FW_REQUIRE(proj_stride >= channels && beta_col >= 0 && beta_col + heads <= proj_stride,
                "delta_prepare: the projections' rows (%d wide) do not hold %d channels and %d strengths at %d", proj_stride, channels, heads, beta_col);
+    FW_REQUIRE(a_stride >= heads * dim, "delta_prepare: the decays' arguments (%d wide) do not hold %d x %d", a_stride, heads, dim);
     FW_REQUIRE(rows <= 1 << 20 && segments <= 65535 && 2 * kv_heads + 2 * heads <= 65535, "delta_prepare: too many rows, segments or heads");
     if (rows == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
     dim3 grid(rows, 2 * kv_heads + 2 * heads);
     dim3 state_grid((channels + 127) / 128, segments);
+    const bool single = rows == segments;       // every segment one row: the memory moves on inside the one kernel
+#define FW_PREPARE_LAUNCH(TI, SINGLE)                                                                                         \
+    delta_prepare_kernel<TI, SINGLE><<<grid, 64, 0, s>>>((const TI*)proj, proj_stride, beta_col, (const TI*)a, a_stride, taps, \
+                                                         conv_state, A_log, dt_bias, row_seg, seg_row0, seg_slot, records,     \
+                                                         heads, kv_heads, dim, vdim, taps_count)
     if (dtype == FW_F32) {
-        delta_prepare_kernel<float><<<grid, 64, 0, s>>>((const float*)proj, proj_stride, beta_col, (const float*)a, taps, conv_state, A_log,
-                                                        dt_bias, row_seg, seg_row0, seg_slot, qkv_out, decay_out, beta_out, heads,
-                                                        kv_heads, dim, vdim, taps_count);
-        if (taps_count > 1)
+        if (single) FW_PREPARE_LAUNCH(float, true);
+        else FW_PREPARE_LAUNCH(float, false);
+        if (taps_count > 1 && !single)
             conv_state_kernel<float><<<state_grid, 128, 0, s>>>((const float*)proj, proj_stride, conv_state, seg_row0, seg_slot, channels, taps_count);
     } else if (dtype == FW_BF16) {
-        delta_prepare_kernel<bf16_t><<<grid, 64, 0, s>>>((const bf16_t*)proj, proj_stride, beta_col, (const bf16_t*)a, taps, conv_state, A_log,
-                                                         dt_bias, row_seg, seg_row0, seg_slot, qkv_out, decay_out, beta_out, heads,
-                                                         kv_heads, dim, vdim, taps_count);
-        if (taps_count > 1)
+        if (single) FW_PREPARE_LAUNCH(bf16_t, true);
+        else FW_PREPARE_LAUNCH(bf16_t, false);
+        if (taps_count > 1 && !single)
             conv_state_kernel<bf16_t><<<state_grid, 128, 0, s>>>((const bf16_t*)proj, proj_stride, conv_state, seg_row0, seg_slot, channels, taps_count);
     } else {
         FW_REQUIRE(false, "delta_prepare: unknown dtype %d", dtype);
     }
+#undef FW_PREPARE_LAUNCH
     FW_LAUNCH_CHECK("delta_prepare");
     return 0;
 }
 
 // ---- the recurrence -----------------------------------------------------------------------------
+extern "C" int fw_delta_record_floats(int dim, int vdim) { return 3 * ((dim + 3) & ~3) + 4 + ((vdim + 3) & ~3); }
+
 // Workgroup (segment, head, block of 64 value channels); thread = 4 * column + quarter. RPT: rows of
-// a column per thread; the column's rows quarter * RPT .. + RPT - 1 (rows from dim on hold zeros).
-// LDS per staged token: q, k, g (4 * RPT each, zero filled past dim), then the block's 64 values,
-// then beta.
+// a column per thread, the column's rows quarter * RPT .. + RPT - 1 (rows from dim on hold zeros).
+// LDS per staged token: q, k, g (4 * RPT each; past the record's padded dim they stay zero), beta and
+// three unused, then the block's 64 values. A thread copies the same pieces of every chunk (16-byte
+// pieces: where each lies in a token's record and in LDS is worked out once).
 template <int RPT>
 __global__ __launch_bounds__(256) void gated_delta_rule_kernel(
-    const float* __restrict__ qkv, const float* __restrict__ decay, const float* __restrict__ beta,
-    float* __restrict__ state, float* __restrict__ out, const int32_t* __restrict__ seg_row0,
-    const int32_t* __restrict__ seg_slot, int heads, int kv_heads, int dim, int vdim) {
+    const float* __restrict__ records, float* __restrict__ state, float* __restrict__ out,
+    const int32_t* __restrict__ seg_row0, const int32_t* __restrict__ seg_slot, int heads, int dim, int vdim) {
+    typedef __attribute__((ext_vector_type(4))) float f32x4;
     constexpr int DP = 4 * RPT;
-    constexpr int TOKEN = 3 * DP + DELTA_COLUMNS + 4;
+    constexpr int TOKEN = 3 * DP + 4 + DELTA_COLUMNS;
+    constexpr int PIECES = (DELTA_CHUNK * (TOKEN / 4) + 255) / 256;      // 16-byte pieces of a chunk per thread, at most
     __shared__ __attribute__((aligned(16))) float staged[DELTA_CHUNK * TOKEN];
     const int seg = blockIdx.x, head = blockIdx.y, block = blockIdx.z;
-    const int kvh = head / (heads / kv_heads);
     const int column = block * DELTA_COLUMNS + threadIdx.x / 4, quarter = threadIdx.x % 4;
     const bool live = column < vdim;
     const int first = seg_row0[seg], count = seg_row0[seg + 1] - first;
-    const int conv_channels = 2 * kv_heads * dim + heads * vdim;
+    const int d4 = (dim + 3) & ~3, v4 = (vdim + 3) & ~3;
+    const int record = 3 * d4 + 4 + v4;
+    const int values_here = v4 - block * DELTA_COLUMNS < DELTA_COLUMNS ? v4 - block * DELTA_COLUMNS : DELTA_COLUMNS;
+    const int per_token = (3 * d4 + 4 + values_here) / 4;                // pieces of a token that this block needs
+    // this thread's pieces: token of the chunk, place in the record, place in LDS (-1: none)
+    int piece_token[PIECES], piece_from[PIECES], piece_to[PIECES];
+#pragma unroll
+    for (int i = 0; i < PIECES; ++i) {
+        const int item = threadIdx.x + 256 * i;
+        const int token = item / per_token, f = (item % per_token) * 4;
+        piece_token[i] = token < DELTA_CHUNK ? token : DELTA_CHUNK;
+        int from, to;
+        if (f < 3 * d4) {
+            const int which = f / d4, within = f % d4;
+            from = f;
+            to = which * DP + within;
+        } else if (f == 3 * d4) {
+            from = f;
+            to = 3 * DP;
+        } else {
+            from = 3 * d4 + 4 + block * DELTA_COLUMNS + (f - 3 * d4 - 4);
+            to = 3 * DP + 4 + (f - 3 * d4 - 4);
+        }
+        piece_from[i] = from;
+        piece_to[i] = token * TOKEN + to;
+    }
+    for (int i = threadIdx.x; i < DELTA_CHUNK * TOKEN; i += 256) staged[i] = 0.0f;
+    const float* source = records + ((size_t)first * heads + head) * record;
+    const size_t token_stride = (size_t)heads * record;
+    f32x4 held[PIECES];
+    auto ask = [&](int base) {
+        const int tokens = count - base < DELTA_CHUNK ? count - base : DELTA_CHUNK;
+#pragma unroll
+        for (int i = 0; i < PIECES; ++i)
+            if (piece_token[i] < tokens)
+                held[i] = *reinterpret_cast<const f32x4*>(source + (size_t)(base + piece_token[i]) * token_stride + piece_from[i]);
+    };
+    auto put = [&](int base) {
+        const int tokens = count - base < DELTA_CHUNK ? count - base : DELTA_CHUNK;
+#pragma unroll
+        for (int i = 0; i < PIECES; ++i)
+            if (piece_token[i] < tokens) *reinterpret_cast<f32x4*>(staged + piece_to[i]) = held[i];
+    };
+    ask(0);
     float* mine = state + (((size_t)seg_slot[seg] * heads + head) * vdim + (live ? column : 0)) * dim;
     float S[RPT];
 #pragma unroll
@@ -171,35 +239,20 @@ __global__ __launch_bounds__(256) void gated_delta_rule_kernel(
         const int i = quarter * RPT + t;
         S[t] = (live && i < dim) ? mine[i] : 0.0f;
     }
+    __syncthreads();        // the zeros are in place
+    put(0);
+    __syncthreads();
     for (int base = 0; base < count; base += DELTA_CHUNK) {
         const int tokens = count - base < DELTA_CHUNK ? count - base : DELTA_CHUNK;
-        __syncthreads();
-        for (int item = threadIdx.x; item < tokens * TOKEN; item += 256) {
-            const int token = item / TOKEN, at = item % TOKEN;
-            const size_t row = (size_t)first + base + token;
-            float value = 0.0f;
-            if (at < DP) {
-                if (at < dim) value = qkv[row * conv_channels + kvh * dim + at];
-            } else if (at < 2 * DP) {
-                if (at - DP < dim) value = qkv[row * conv_channels + (kv_heads + kvh) * dim + (at - DP)];
-            } else if (at < 3 * DP) {
-                if (at - 2 * DP < dim) value = decay[(row * heads + head) * dim + (at - 2 * DP)];
-            } else if (at < 3 * DP + DELTA_COLUMNS) {
-                const int c = block * DELTA_COLUMNS + (at - 3 * DP);
-                if (c < vdim) value = qkv[row * conv_channels + 2 * kv_heads * dim + head * vdim + c];
-            } else if (at == 3 * DP + DELTA_COLUMNS) {
-                value = beta[row * heads + head];
-            }
-            staged[item] = value;
-        }
-        __syncthreads();
+        const bool more = base + DELTA_CHUNK < count;
+        if (more) ask(base + DELTA_CHUNK);
         for (int token = 0; token < tokens; ++token) {
             const float* t0 = staged + token * TOKEN;
             const float* qs = t0 + quarter * RPT;
             const float* ks = t0 + DP + quarter * RPT;
             const float* gs = t0 + 2 * DP + quarter * RPT;
-            const float v = t0[3 * DP + threadIdx.x / 4];
-            const float b = t0[3 * DP + DELTA_COLUMNS];
+            const float b = t0[3 * DP];
+            const float v = t0[3 * DP + 4 + threadIdx.x / 4];
             float seen = 0.0f;
 #pragma unroll
             for (int t = 0; t < RPT; ++t) {
@@ -219,6 +272,9 @@ __global__ __launch_bounds__(256) void gated_delta_rule_kernel(
             read += __shfl_xor(read, 2, 64);
             if (live && quarter == 0) out[((size_t)first + base + token) * heads * vdim + head * vdim + column] = read;
         }
+        __syncthreads();
+        if (more) put(base + DELTA_CHUNK);
+        __syncthreads();
     }
     if (live) {
 #pragma unroll
@@ -229,18 +285,18 @@ __global__ __launch_bounds__(256) void gated_delta_rule_kernel(
     }
 }
 
-extern "C" int fw_gated_delta_rule(const float* qkv, const float* decay, const float* beta, float* state, float* out,
-                                   const int32_t* seg_row0, const int32_t* seg_slot, int rows, int segments, int heads,
-                                   int kv_heads, int dim, int vdim, int slots, void* stream) {
-    FW_REQUIRE(rows >= 0 && segments >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0,
-               "gated_delta_rule: heads %d must be a positive multiple of kv heads %d", heads, kv_heads);
+extern "C" int fw_gated_delta_rule(const float* records, float* state, float* out, const int32_t* seg_row0,
+                                   const int32_t* seg_slot, int rows, int segments, int heads, int dim, int vdim,
+                                   int slots, void* stream) {
+    FW_REQUIRE(rows >= 0 && segments >= 0 && heads > 0, "gated_delta_rule: bad sizes rows=%d segments=%d heads=%d", rows, segments, heads);
     FW_REQUIRE(dim > 0 && dim <= 256 && vdim > 0, "gated_delta_rule: dim %d must lie in 1..256 and vdim %d be positive", dim, vdim);
     FW_REQUIRE(slots > 0 && segments <= 65535 && heads <= 65535, "gated_delta_rule: too many segments or heads, or no slots");
+    FW_REQUIRE((uintptr_t)records % 16 == 0, "gated_delta_rule: the records must lie at a multiple of 16 bytes");
     if (rows == 0 || segments == 0) return 0;
     dim3 grid(segments, heads, (vdim + DELTA_COLUMNS - 1) / DELTA_COLUMNS);
     hipStream_t s = (hipStream_t)stream;
 #define FW_DELTA_LAUNCH(RPT) \
-    gated_delta_rule_kernel<RPT><<<grid, 256, 0, s>>>(qkv, decay, beta, state, out, seg_row0, seg_slot, heads, kv_heads, dim, vdim)
+    gated_delta_rule_kernel<RPT><<<grid, 256, 0, s>>>(records, state, out, seg_row0, seg_slot, heads, dim, vdim)
     if (dim <= 16) FW_DELTA_LAUNCH(4);
     else if (dim <= 32) FW_DELTA_LAUNCH(8);
     else if (dim <= 64) FW_DELTA_LAUNCH(16);

@@ -202,25 +202,28 @@ int fw_fill_zero(void* ptr, long long bytes, void* stream);
 int fw_fill_zero_pieces(void* ptr, int pieces, long long bytes, long long stride_bytes, void* stream);
 
 // ---- the gated delta rule (a linear recurrence over a matrix state per head) -----------------------
-// What the recurrence reads, from one step's projections. proj [rows][proj_stride]: columns
-// 0 .. 2 G d + H vd - 1 hold q | k | v before their short causal convolutions (G = kv_heads heads of d
-// = dim channels for q and for k, H = heads of vd = vdim channels for v), columns beta_col .. + H - 1
-// the write strengths before their sigmoid. a [rows][H d]: the decays' arguments. taps [channels][L],
-// the last column the current token's; conv_state [slots][channels][L - 1], oldest first, read and
-// then moved on by the segment's rows. qkv_out [rows][channels]: silu of the convolutions, q and k of
-// unit length per head (sum of squares + 1e-6 under the root), q also times d^-1/2. decay_out
-// [rows][H d] = exp(-exp(A_log[h]) * softplus(a + dt_bias)); beta_out [rows][H].
-int fw_delta_prepare(const void* proj, int dtype, int proj_stride, int beta_col, const void* a, const float* taps,
+// What the recurrence reads, from one step's projections, as one record per (row, head):
+// [q (d4) | k (d4) | g (d4) | beta, 3 unused | v (v4)] float32, d4 and v4 the head sizes rounded up to a
+// multiple of 4 (fw_delta_record_floats floats in all; what lies past dim or vdim is zero).
+// proj [rows][proj_stride]: columns 0 .. 2 G d + H vd - 1 hold q | k | v before their short causal
+// convolutions (G = kv_heads heads of d = dim channels for q and for k, H = heads of vd = vdim channels
+// for v; head h reads q/k head h / (H / G)), columns beta_col .. + H - 1 the write strengths before
+// their sigmoid. a [rows][a_stride]: the decays' arguments in its first H d columns. taps
+// [channels][L], the last column the current token's; conv_state [slots][channels][L - 1], oldest
+// first, read and then moved on by the segment's rows. q, k, v are the silu of the convolutions, q and
+// k of unit length per head (sum of squares + 1e-6 under the root), q also times d^-1/2;
+// g = exp(-exp(A_log[h]) * softplus(a + dt_bias)).
+int fw_delta_record_floats(int dim, int vdim);
+int fw_delta_prepare(const void* proj, int dtype, int proj_stride, int beta_col, const void* a, int a_stride, const float* taps,
                      float* conv_state, const float* A_log, const float* dt_bias, const int32_t* row_seg,
-                     const int32_t* seg_row0, const int32_t* seg_slot, float* qkv_out, float* decay_out,
-                     float* beta_out, int rows, int segments, int heads, int kv_heads, int dim, int vdim,
-                     int taps_count, int slots, void* stream);
+                     const int32_t* seg_row0, const int32_t* seg_slot, float* records, int rows, int segments,
+                     int heads, int kv_heads, int dim, int vdim, int taps_count, int slots, void* stream);
 // Per segment and head, token by token: S <- diag(g) S; u = beta (v - S^T k); S <- S + k u^T;
-// o = S^T q. state [slots][H][vd][d] (S transposed), read at the segment's start and written at its
-// end. out [rows][H vd]. Head h reads q/k head h / (H / G).
-int fw_gated_delta_rule(const float* qkv, const float* decay, const float* beta, float* state, float* out,
-                        const int32_t* seg_row0, const int32_t* seg_slot, int rows, int segments, int heads,
-                        int kv_heads, int dim, int vdim, int slots, void* stream);
+// o = S^T q. records [rows][H][fw_delta_record_floats]. state [slots][H][vd][d] (S transposed), read
+// at the segment's start and written at its end. out [rows][H vd].
+int fw_gated_delta_rule(const float* records, float* state, float* out, const int32_t* seg_row0,
+                        const int32_t* seg_slot, int rows, int segments, int heads, int dim, int vdim,
+                        int slots, void* stream);
 // out[r][h][j] = o[r][h][j] * rsqrt(mean_j o[r][h]^2 + eps) * weight[j] * sigmoid(gate[r][h vd + j])
 int fw_gated_head_norm(const float* o, const void* gate, int gate_dtype, int gate_stride, const float* weight,
                        void* out, int out_dtype, int rows, int heads, int vdim, float eps, void* stream);

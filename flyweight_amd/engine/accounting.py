@@ -69,16 +69,30 @@ def attention_flops(model, rows: int, keys_before: int = 0) -> int:
     paged cache (2 products x 2 flops x heads x head size per visible query-key pair; a window
     bounds the pairs)."""
     total = 0
+
+    def mixers_of(part):
+        """A mixer, or the mixers it is made of."""
+        below = part.sub_parts() if hasattr(part, "sub_parts") else ()
+        if not below:
+            yield part
+        for inner in below:
+            yield from mixers_of(inner)
+
     for entry in model.spec.schedule:
-        mixer = getattr(model.layers[entry.layer], "mixer", None)
-        need = mixer.cache_need() if mixer is not None else None
-        if need is None or not need.paged or not hasattr(mixer, "num_heads"):
-            continue
-        pairs = 0
-        for row in range(rows):
-            visible = keys_before + row + 1
-            pairs += min(visible, need.window) if need.window else visible
-        total += 4 * mixer.num_heads * mixer.head_dim * pairs
+        top = getattr(model.layers[entry.layer], "mixer", None)
+        for mixer in (mixers_of(top) if top is not None else ()):
+            if hasattr(mixer, "mixing_flops"):      # a mixer that is no attention says what its rows cost
+                total += mixer.mixing_flops(rows, keys_before)
+                continue
+            need = mixer.cache_need()
+            if need is None or isinstance(need, dict) or not need.paged or not hasattr(mixer, "num_heads"):
+                continue
+            if need.window:     # visible keys of row r: min(keys_before + r + 1, window)
+                full = max(0, min(rows, need.window - keys_before - 1))     # rows that still see fewer than a window
+                pairs = full * keys_before + full * (full + 1) // 2 + (rows - full) * need.window
+            else:
+                pairs = rows * keys_before + rows * (rows + 1) // 2
+            total += 2 * mixer.num_heads * (mixer.head_dim + getattr(mixer, "v_head_dim", mixer.head_dim)) * pairs
     return total
 
 

@@ -144,6 +144,14 @@ def _dev(*tensors: Optional[torch.Tensor]) -> None:
             raise KernelError("kernels need contiguous tensors")
 
 
+def _dev_rows(t: torch.Tensor, name: str) -> None:
+    """A matrix whose rows may lie apart (a view of some columns of wider rows), each row contiguous."""
+    if not t.is_cuda:
+        raise KernelError("kernels run on the GPU only; got a CPU tensor")
+    if t.dim() != 2 or t.stride(1) != 1:
+        raise KernelError(f"{name} must be a matrix with contiguous rows")
+
+
 def _p(t: Optional[torch.Tensor]) -> ctypes.c_void_p:
     return ctypes.c_void_p(0 if t is None else t.data_ptr())
 
@@ -1027,15 +1035,17 @@ def delta_prepare(proj: torch.Tensor, beta_col: int, a: torch.Tensor, taps: torc
     its first ``channels`` = 2 kv_heads dim + heads vdim columns are q | k | v before their short
     convolutions, columns ``beta_col`` .. + heads the write strengths before the sigmoid; ``a``
     [rows, heads dim] the decays' arguments. ``conv_state`` [slots, channels, taps - 1] is read and
-    moved on. Returns float32 (qkv [rows, channels], decay [rows, heads dim], beta [rows, heads])."""
-    _dev(proj, a, taps, conv_state, A_log, dt_bias, row_seg, seg_row0, seg_slot)
+    moved on. Returns float32 records [rows, heads, delta_record_floats(dim, vdim)]: per row and head
+    q | k | g | beta | v as the recurrence reads them (q and k of the head's group)."""
+    _dev(proj, taps, conv_state, A_log, dt_bias, row_seg, seg_row0, seg_slot)
+    _dev_rows(a, "a")
     rows, stride = proj.shape
     channels = 2 * kv_heads * dim + heads * vdim
     count = taps.shape[1]
-    if proj.dtype != a.dtype or not proj.is_contiguous() or not a.is_contiguous():
-        raise KernelError("delta_prepare: the projections and the decays' arguments come in one dtype, contiguous")
+    if proj.dtype != a.dtype or not proj.is_contiguous() or a.dim() != 2 or a.stride(1) != 1:
+        raise KernelError("delta_prepare: the projections and the decays' arguments come in one dtype, rows contiguous")
     if a.shape != (rows, heads * dim):
-        raise KernelError(f"delta_prepare: a is {tuple(a.shape)}, expected {(rows, heads * dim)}")
+        raise KernelError(f"delta_prepare: a is {tuple(a.shape)}, expected {(rows, heads * dim)} (a view of wider rows will do)")
     for name, t, shape in (("taps", taps, (channels, count)), ("A_log", A_log, (heads,)), ("dt_bias", dt_bias, (heads * dim,))):
         _want(t, torch.float32, name)
         if t.shape != shape or not t.is_contiguous():
@@ -1047,26 +1057,29 @@ def delta_prepare(proj: torch.Tensor, beta_col: int, a: torch.Tensor, taps: torc
         _want(t, torch.int32, name)
         if t.numel() < n:
             raise KernelError(f"delta_prepare: {name} holds {t.numel()} entries, needs {n}")
-    qkv = torch.empty((rows, channels), dtype=torch.float32, device=proj.device)
-    decay = torch.empty((rows, heads * dim), dtype=torch.float32, device=proj.device)
-    beta = torch.empty((rows, heads), dtype=torch.float32, device=proj.device)
-    _check(library().fw_delta_prepare(_p(proj), _code(proj.dtype), stride, int(beta_col), _p(a), _p(taps), _p(conv_state), _p(A_log),
-                                      _p(dt_bias), _p(row_seg), _p(seg_row0), _p(seg_slot), _p(qkv), _p(decay), _p(beta), rows,
-                                      int(segments), heads, kv_heads, dim, vdim, count, conv_state.shape[0], _stream()))
-    return qkv, decay, beta
+    records = torch.empty((rows, heads, delta_record_floats(dim, vdim)), dtype=torch.float32, device=proj.device)
+    _check(library().fw_delta_prepare(_p(proj), _code(proj.dtype), stride, int(beta_col), _p(a), a.stride(0) if rows > 1 else heads * dim,
+                                      _p(taps), _p(conv_state), _p(A_log), _p(dt_bias), _p(row_seg), _p(seg_row0), _p(seg_slot),
+                                      _p(records), rows, int(segments), heads, kv_heads, dim, vdim, count, conv_state.shape[0], _stream()))
+    return records
 
 
-def gated_delta_rule(qkv: torch.Tensor, decay: torch.Tensor, beta: torch.Tensor, state: torch.Tensor, seg_row0: torch.Tensor,
-                     seg_slot: torch.Tensor, segments: int, heads: int, kv_heads: int, dim: int, vdim: int) -> torch.Tensor:
-    """The recurrence over each segment's rows; ``state`` [slots, heads, vdim, dim] float32 (the
-    matrix transposed) is read at a segment's start and written at its end. Returns [rows, heads vdim]."""
-    _dev(qkv, decay, beta, state, seg_row0, seg_slot)
-    rows = qkv.shape[0]
-    for name, t, shape in (("qkv", qkv, (rows, 2 * kv_heads * dim + heads * vdim)), ("decay", decay, (rows, heads * dim)),
-                           ("beta", beta, (rows, heads))):
-        _want(t, torch.float32, name)
-        if t.shape != shape or not t.is_contiguous():
-            raise KernelError(f"gated_delta_rule: {name} is {tuple(t.shape)}, expected {shape}")
+def delta_record_floats(dim: int, vdim: int) -> int:
+    """Floats of what one token brings to one head of the recurrence: q | k | g (dim rounded up to a
+    multiple of 4 each) | beta and three unused | v (vdim rounded up likewise)."""
+    return 3 * ((dim + 3) // 4 * 4) + 4 + (vdim + 3) // 4 * 4
+
+
+def gated_delta_rule(records: torch.Tensor, state: torch.Tensor, seg_row0: torch.Tensor, seg_slot: torch.Tensor,
+                     segments: int, heads: int, dim: int, vdim: int) -> torch.Tensor:
+    """The recurrence over each segment's rows. ``records`` [rows, heads, delta_record_floats]: what
+    ``delta_prepare`` made. ``state`` [slots, heads, vdim, dim] float32 (the matrix transposed) is read
+    at a segment's start and written at its end. Returns [rows, heads vdim]."""
+    _dev(records, state, seg_row0, seg_slot)
+    rows = records.shape[0]
+    _want(records, torch.float32, "records")
+    if records.shape != (rows, heads, delta_record_floats(dim, vdim)) or not records.is_contiguous():
+        raise KernelError(f"gated_delta_rule: records are {tuple(records.shape)}, expected {(rows, heads, delta_record_floats(dim, vdim))}")
     _want(state, torch.float32, "state")
     if state.dim() != 4 or state.shape[1:] != (heads, vdim, dim) or not state.is_contiguous():
         raise KernelError(f"gated_delta_rule: the state is {tuple(state.shape)}, expected [slots, {heads}, {vdim}, {dim}]")
@@ -1074,24 +1087,25 @@ def gated_delta_rule(qkv: torch.Tensor, decay: torch.Tensor, beta: torch.Tensor,
         _want(t, torch.int32, name)
         if t.numel() < n:
             raise KernelError(f"gated_delta_rule: {name} holds {t.numel()} entries, needs {n}")
-    out = torch.empty((rows, heads * vdim), dtype=torch.float32, device=qkv.device)
-    _check(library().fw_gated_delta_rule(_p(qkv), _p(decay), _p(beta), _p(state), _p(out), _p(seg_row0), _p(seg_slot), rows,
-                                         int(segments), heads, kv_heads, dim, vdim, state.shape[0], _stream()))
+    out = torch.empty((rows, heads * vdim), dtype=torch.float32, device=records.device)
+    _check(library().fw_gated_delta_rule(_p(records), _p(state), _p(out), _p(seg_row0), _p(seg_slot), rows, int(segments), heads,
+                                         dim, vdim, state.shape[0], _stream()))
     return out
 
 
 def gated_head_norm(o: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, heads: int, vdim: int, eps: float,
                     out_dtype: torch.dtype) -> torch.Tensor:
     """Per head: o / rms(o) * weight * sigmoid(gate); ``o`` float32 [rows, heads vdim], ``gate``
-    [rows, heads vdim] (float32, or bfloat16 beside a bfloat16 output)."""
-    _dev(o, gate, weight)
+    [rows, heads vdim] (float32, or bfloat16 beside a bfloat16 output; a view of wider rows will do)."""
+    _dev(o, weight)
+    _dev_rows(gate, "gate")
     _want(o, torch.float32, "o")
     _want(weight, torch.float32, "weight")
     rows = o.shape[0]
-    if o.shape != (rows, heads * vdim) or gate.shape != o.shape or weight.shape != (vdim,) or not o.is_contiguous() or not gate.is_contiguous():
+    if o.shape != (rows, heads * vdim) or gate.shape != o.shape or weight.shape != (vdim,) or not o.is_contiguous() or gate.stride(1) != 1:
         raise KernelError(f"gated_head_norm: o {tuple(o.shape)}, gate {tuple(gate.shape)}, weight {tuple(weight.shape)} do not fit {heads} x {vdim}")
     out = torch.empty((rows, heads * vdim), dtype=out_dtype, device=o.device)
-    _check(library().fw_gated_head_norm(_p(o), _p(gate), _code(gate.dtype), heads * vdim, _p(weight), _p(out), _code(out_dtype), rows,
+    _check(library().fw_gated_head_norm(_p(o), _p(gate), _code(gate.dtype), gate.stride(0) if rows > 1 else heads * vdim, _p(weight), _p(out), _code(out_dtype), rows,
                                         heads, vdim, ctypes.c_float(eps), _stream()))
     return out
 

@@ -65,6 +65,11 @@ class GatedDeltaRule(Mixer):
     def _name(self, which: str) -> str:
         return self.prefix + self.names[which]
 
+    def mixing_flops(self, rows: int, keys_before: int = 0) -> int:
+        """Flops of the recurrence itself: per token and head three passes over the state (decay and
+        read with the key, write, read with the query), a multiply and an add each."""
+        return 6 * self.heads * self.dim * self.vdim * rows
+
     def tensors(self) -> Dict[str, TensorDecl]:
         D, H, G, d, dv, L = self.hidden, self.heads, self.kv_heads, self.dim, self.vdim, self.taps_count
         return {
@@ -82,14 +87,19 @@ class GatedDeltaRule(Mixer):
     def bind(self, tensors, dtype, device) -> None:
         super().bind(tensors, dtype, device)
         t = {which: tensors[self._name(which)] for which in self.names}
-        # one operand for everything that reads h: q | k | v (the convolutions' inputs), the write
-        # strengths, and the inner halves of the two low-rank maps
+        # One operand for what the recurrence reads of h in float32: q | k | v (the convolutions' inputs)
+        # and the write strengths. The two low-rank maps share their two products: the inner halves
+        # side by side (their activations leave in the activation dtype, as any product's input), and
+        # the outer halves as one block-diagonal operand whose zeros add nothing, so that one product
+        # gives the decays' arguments and the gates side by side.
         self.beta_col = self.channels
-        self.a_col = self.beta_col + self.heads
-        self.g_col = self.a_col + self.rank_a
-        self.in_proj = Linear(torch.cat([t["q"], t["k"], t["v"], t["b"], t["a1"], t["g1"]], dim=0))
-        self.a2 = Linear(t["a2"])
-        self.g2 = Linear(t["g2"])
+        self.in_proj = Linear(torch.cat([t["q"], t["k"], t["v"], t["b"]], dim=0))
+        self.low = Linear(torch.cat([t["a1"], t["g1"]], dim=0))
+        a2, g2 = t["a2"], t["g2"]
+        outer = torch.zeros((a2.shape[0] + g2.shape[0], self.rank_a + self.rank_g), dtype=a2.dtype, device=a2.device)
+        outer[:a2.shape[0], :self.rank_a] = a2
+        outer[a2.shape[0]:, self.rank_a:] = g2
+        self.outer = Linear(outer)
         self.out = Linear(t["o"])
         self.taps = torch.cat([t["q_conv"], t["k_conv"], t["v_conv"]], dim=0).contiguous()
         self.A_log, self.dt_bias, self.norm_weight = t["A_log"], t["dt_bias"], t["norm"]
@@ -106,14 +116,13 @@ class GatedDeltaRule(Mixer):
         """The heads' normed and gated read-outs [rows, heads * vdim] in the activation dtype; the
         request's state moves on by the step's rows."""
         proj = self.in_proj.forward(h, out_dtype=torch.float32)
-        # the low-rank maps' inner activations pass in the activation dtype, as any product's input
-        a = self.a2.forward(ops.round_rows(proj[:, self.a_col:self.g_col].contiguous(), self.dtype), out_dtype=torch.float32)
-        gate = self.g2.forward(ops.round_rows(proj[:, self.g_col:].contiguous(), self.dtype), out_dtype=torch.float32)
-        qkv, decay, beta = ops.delta_prepare(proj, self.beta_col, a, self.taps, self._conv_state(cache), self.A_log, self.dt_bias,
-                                             ctx.row_seg, ctx.seg_row0, ctx.seg_slot, ctx.num_segments, self.heads, self.kv_heads,
-                                             self.dim, self.vdim)
-        o = ops.gated_delta_rule(qkv, decay, beta, cache["state"].state, ctx.seg_row0, ctx.seg_slot, ctx.num_segments,
-                                 self.heads, self.kv_heads, self.dim, self.vdim)
+        both = self.outer.forward(self.low.forward(h), out_dtype=torch.float32)
+        a, gate = both[:, :self.heads * self.dim], both[:, self.heads * self.dim:]
+        records = ops.delta_prepare(proj, self.beta_col, a, self.taps, self._conv_state(cache), self.A_log, self.dt_bias,
+                                    ctx.row_seg, ctx.seg_row0, ctx.seg_slot, ctx.num_segments, self.heads, self.kv_heads,
+                                    self.dim, self.vdim)
+        o = ops.gated_delta_rule(records, cache["state"].state, ctx.seg_row0, ctx.seg_slot, ctx.num_segments,
+                                 self.heads, self.dim, self.vdim)
         return ops.gated_head_norm(o, gate, self.norm_weight, self.heads, self.vdim, self.eps, self.dtype)
 
     def output(self, h, ctx, cache) -> torch.Tensor:

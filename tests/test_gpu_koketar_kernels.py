@@ -21,6 +21,13 @@ def ints(values):
     return torch.tensor(list(values), dtype=torch.int32, device="cuda")
 
 
+def record_layout(dim, vdim):
+    """Where q, k, g, beta and v lie in what a token brings to a head: each of q, k, g and v rounded up
+    to a multiple of four floats, beta and three unused floats in front of v."""
+    d4, v4 = (dim + 3) // 4 * 4, (vdim + 3) // 4 * 4
+    return {"q": 0, "k": d4, "g": 2 * d4, "beta": 3 * d4, "v": 3 * d4 + 4, "floats": 3 * d4 + 4 + v4}
+
+
 @pytest.mark.parametrize("heads,kv_heads,dim,vdim", [(3, 1, 20, 70), (2, 2, 64, 64), (4, 2, 8, 5), (1, 1, 130, 129), (2, 1, 256, 16)])
 def test_recurrence_over_segments_with_carried_state(heads, kv_heads, dim, vdim):
     from flyweight_amd.kernels import ops
@@ -35,10 +42,19 @@ def test_recurrence_over_segments_with_carried_state(heads, kv_heads, dim, vdim)
     decay[:, 0, ::2] = 1.0                                      # channels that never forget
     start = rng.normal(size=(5, heads, dim, vdim))              # five slots, S[slot, head] as the equations write it
     state = dev(start.transpose(0, 1, 3, 2))                    # stored transposed
-    qkv = np.concatenate([q.reshape(rows, -1), k.reshape(rows, -1), v.reshape(rows, -1)], axis=1)
+    at = record_layout(dim, vdim)
+    assert at["floats"] == ops.delta_record_floats(dim, vdim)
+    records = np.zeros((rows, heads, at["floats"]))
+    for head in range(heads):
+        g = head // (heads // kv_heads)
+        records[:, head, at["q"]:at["q"] + dim] = q[:, g]
+        records[:, head, at["k"]:at["k"] + dim] = k[:, g]
+        records[:, head, at["g"]:at["g"] + dim] = decay[:, head]
+        records[:, head, at["beta"]] = beta[:, head]
+        records[:, head, at["v"]:at["v"] + vdim] = v[:, head]
     seg_row0 = np.concatenate([[0], np.cumsum(lengths)])
-    out = ops.gated_delta_rule(dev(qkv), dev(decay.reshape(rows, -1)), dev(beta), state, ints(seg_row0), ints(slots_of),
-                               len(lengths), heads, kv_heads, dim, vdim).cpu().numpy().reshape(rows, heads, vdim)
+    out = ops.gated_delta_rule(dev(records), state, ints(seg_row0), ints(slots_of), len(lengths), heads, dim,
+                               vdim).cpu().numpy().reshape(rows, heads, vdim)
     after = state.cpu().numpy().transpose(0, 1, 3, 2)
     for seg, (length, slot) in enumerate(zip(lengths, slots_of)):
         for head in range(heads):
@@ -72,10 +88,20 @@ def test_what_the_recurrence_reads(taps):
     conv_state = dev(memory)
     seg_row0 = np.concatenate([[0], np.cumsum(lengths)])
     row_seg = np.repeat(np.arange(len(lengths)), lengths)
-    qkv, decay, beta = ops.delta_prepare(dev(proj), channels, dev(a), dev(np.concatenate([w["q.conv"], w["k.conv"], w["v.conv"]])),
-                                         conv_state, dev(A_log), dev(dt_bias), ints(row_seg), ints(seg_row0), ints(slots_of),
-                                         len(lengths), heads, kv_heads, dim, vdim)
-    qkv, decay, beta, after = qkv.cpu().numpy(), decay.cpu().numpy(), beta.cpu().numpy(), conv_state.cpu().numpy()
+    wide = dev(np.concatenate([a, rng.normal(size=(rows, 5))], axis=1))      # the arguments as a view of wider rows
+    records = ops.delta_prepare(dev(proj), channels, wide[:, :heads * dim], dev(np.concatenate([w["q.conv"], w["k.conv"], w["v.conv"]])),
+                                conv_state, dev(A_log), dev(dt_bias), ints(row_seg), ints(seg_row0), ints(slots_of),
+                                len(lengths), heads, kv_heads, dim, vdim).cpu().numpy()
+    at = record_layout(dim, vdim)
+    after = conv_state.cpu().numpy()
+    # every head's record holds the q and k of its group (one group here), its own v, decays and strength
+    for head in range(1, heads):
+        np.testing.assert_array_equal(records[:, head, :at["g"]], records[:, 0, :at["g"]])
+    assert (records[:, :, at["q"] + dim:at["k"]] == 0).all() and (records[:, :, at["v"] + vdim:] == 0).all()
+    qkv = np.concatenate([records[:, 0, at["q"]:at["q"] + dim], records[:, 0, at["k"]:at["k"] + dim],
+                          records[:, :, at["v"]:at["v"] + vdim].reshape(rows, -1)], axis=1)
+    decay = records[:, :, at["g"]:at["g"] + dim].reshape(rows, -1)
+    beta = records[:, :, at["beta"]]
     taps_all = np.concatenate([w["q.conv"], w["k.conv"], w["v.conv"]])
     for seg, (length, slot) in enumerate(zip(lengths, slots_of)):
         r0 = seg_row0[seg]
