@@ -5,19 +5,18 @@
 // a value v (vdim channels), a write strength beta and a decay g per key channel:
 //     S <- diag(g) S;   u = beta (v - S^T k);   S <- S + k u^T;   o = S^T q
 // so the read-out sees the token's own write. Columns of S (value channels) never meet: a column is
-// owned by four lanes, each holding a quarter of its rows in registers, and the two sums over the
-// key channels are reductions over those four lanes. A segment's tokens are walked in order. What a
+// owned by sixteen lanes, each holding a sixteenth of its rows in registers, and the two sums over the
+// key channels are reductions over those lanes. A segment's tokens are walked in order. What a
 // token brings to a head lies in one record, [q | k | g | beta | v] (fw_delta_record_floats), so that a
 // chunk of tokens is a plain copy into LDS; the copy of the next chunk is asked for before the work on
 // this one and waits in registers meanwhile.
 //
-// The state is stored transposed, [slot][head][vdim][dim], so that the quarter columns a wave holds
-// are one contiguous piece of memory.
+// The state is stored transposed, [slot][head][vdim][dim], so that the columns a wave holds are one
+// contiguous piece of memory.
 #include "fw_common.h"
 #include "fw_kernels.h"
 
 #define DELTA_CHUNK 16          // tokens staged in LDS at a time
-#define DELTA_COLUMNS 64        // value channels per workgroup (256 threads: four lanes a column)
 
 __device__ __forceinline__ float fw_sigmoid(float x) { return 1.0f / (1.0f + expf(-x)); }
 __device__ __forceinline__ float fw_softplus(float x) { return x > 20.0f ? x : log1pf(expf(x)); }
@@ -170,29 +169,51 @@ extern "C" int fw_delta_prepare(const void* proj, int dtype, int proj_stride, in
 // ---- the recurrence -----------------------------------------------------------------------------
 extern "C" int fw_delta_record_floats(int dim, int vdim) { return 3 * ((dim + 3) & ~3) + 4 + ((vdim + 3) & ~3); }
 
-// Workgroup (segment, head, block of 64 value channels); thread = 4 * column + quarter. RPT: rows of
-// a column per thread, the column's rows quarter * RPT .. + RPT - 1 (rows from dim on hold zeros).
-// LDS per staged token: q, k, g (4 * RPT each; past the record's padded dim they stay zero), beta and
-// three unused, then the block's 64 values. A thread copies the same pieces of every chunk (16-byte
-// pieces: where each lies in a token's record and in LDS is worked out once).
+// A sum over the 16 lanes of a row of the wave (every lane gets it): neighbours, pairs, then the two
+// mirrors, all inside the vector unit (no trip through the LDS crossbar). After each step the lanes
+// that have met hold one value, so the mirrors may stand for the exchanges between quads and halves.
+template <int CTRL>
+__device__ __forceinline__ float delta_dpp(float x) {
+    return __uint_as_float((uint32_t)__builtin_amdgcn_update_dpp(0, (int)__float_as_uint(x), CTRL, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float delta_row_sum(float x) {
+    x += delta_dpp<0xB1>(x);        // quad_perm [1, 0, 3, 2]
+    x += delta_dpp<0x4E>(x);        // quad_perm [2, 3, 0, 1]
+    x += delta_dpp<0x141>(x);       // row_half_mirror
+    x += delta_dpp<0x140>(x);       // row_mirror
+    return x;
+}
+
+// Workgroup (segment, head, block of 16 value channels); thread = 16 * column + part: a column of S
+// is shared out over the 16 lanes of a row of the wave, RPT rows each (rows part * RPT .. + RPT - 1;
+// rows from dim on hold zeros), so that a head is spread over many compute units: the walk along the
+// tokens is one dependent chain per column, and only its width can be bought. LDS per staged token:
+// q, k, g (16 * RPT each; past the record's padded dim they stay zero), beta and three unused, then the
+// block's 16 values. A thread copies the same pieces of every chunk (16-byte pieces: where each lies in
+// a token's record and in LDS is worked out once).
+#define DELTA_LANES 16
+#define DELTA_COLUMNS (256 / DELTA_LANES)
 template <int RPT>
 __global__ __launch_bounds__(256) void gated_delta_rule_kernel(
     const float* __restrict__ records, float* __restrict__ state, float* __restrict__ out,
     const int32_t* __restrict__ seg_row0, const int32_t* __restrict__ seg_slot, int heads, int dim, int vdim) {
     typedef __attribute__((ext_vector_type(4))) float f32x4;
-    constexpr int DP = 4 * RPT;
+    constexpr int DP = DELTA_LANES * RPT;
     constexpr int TOKEN = 3 * DP + 4 + DELTA_COLUMNS;
     constexpr int PIECES = (DELTA_CHUNK * (TOKEN / 4) + 255) / 256;      // 16-byte pieces of a chunk per thread, at most
     __shared__ __attribute__((aligned(16))) float staged[DELTA_CHUNK * TOKEN];
+    __shared__ float results[DELTA_CHUNK * DELTA_COLUMNS];
+    static_assert(DELTA_CHUNK * DELTA_COLUMNS == 256, "a chunk's read-outs are one per thread");
     const int seg = blockIdx.x, head = blockIdx.y, block = blockIdx.z;
-    const int column = block * DELTA_COLUMNS + threadIdx.x / 4, quarter = threadIdx.x % 4;
+    const int local = threadIdx.x / DELTA_LANES, part = threadIdx.x % DELTA_LANES;
+    const int column = block * DELTA_COLUMNS + local;
     const bool live = column < vdim;
     const int first = seg_row0[seg], count = seg_row0[seg + 1] - first;
     const int d4 = (dim + 3) & ~3, v4 = (vdim + 3) & ~3;
     const int record = 3 * d4 + 4 + v4;
     const int values_here = v4 - block * DELTA_COLUMNS < DELTA_COLUMNS ? v4 - block * DELTA_COLUMNS : DELTA_COLUMNS;
     const int per_token = (3 * d4 + 4 + values_here) / 4;                // pieces of a token that this block needs
-    // this thread's pieces: token of the chunk, place in the record, place in LDS (-1: none)
+    // this thread's pieces: token of the chunk, place in the record, place in LDS
     int piece_token[PIECES], piece_from[PIECES], piece_to[PIECES];
 #pragma unroll
     for (int i = 0; i < PIECES; ++i) {
@@ -201,9 +222,8 @@ __global__ __launch_bounds__(256) void gated_delta_rule_kernel(
         piece_token[i] = token < DELTA_CHUNK ? token : DELTA_CHUNK;
         int from, to;
         if (f < 3 * d4) {
-            const int which = f / d4, within = f % d4;
             from = f;
-            to = which * DP + within;
+            to = (f / d4) * DP + f % d4;
         } else if (f == 3 * d4) {
             from = f;
             to = 3 * DP;
@@ -212,9 +232,10 @@ __global__ __launch_bounds__(256) void gated_delta_rule_kernel(
             to = 3 * DP + 4 + (f - 3 * d4 - 4);
         }
         piece_from[i] = from;
-        piece_to[i] = token * TOKEN + to;
+        piece_to[i] = (token < DELTA_CHUNK ? token : 0) * TOKEN + to;
     }
-    for (int i = threadIdx.x; i < DELTA_CHUNK * TOKEN; i += 256) staged[i] = 0.0f;
+    const int staged_tokens = count < DELTA_CHUNK ? count : DELTA_CHUNK;     // a decode step stages one token
+    for (int i = threadIdx.x; i < staged_tokens * TOKEN; i += 256) staged[i] = 0.0f;
     const float* source = records + ((size_t)first * heads + head) * record;
     const size_t token_stride = (size_t)heads * record;
     f32x4 held[PIECES];
@@ -236,7 +257,7 @@ __global__ __launch_bounds__(256) void gated_delta_rule_kernel(
     float S[RPT];
 #pragma unroll
     for (int t = 0; t < RPT; ++t) {
-        const int i = quarter * RPT + t;
+        const int i = part * RPT + t;
         S[t] = (live && i < dim) ? mine[i] : 0.0f;
     }
     __syncthreads();        // the zeros are in place
@@ -246,31 +267,49 @@ __global__ __launch_bounds__(256) void gated_delta_rule_kernel(
         const int tokens = count - base < DELTA_CHUNK ? count - base : DELTA_CHUNK;
         const bool more = base + DELTA_CHUNK < count;
         if (more) ask(base + DELTA_CHUNK);
-        for (int token = 0; token < tokens; ++token) {
+        // a token's operands are read from LDS while the token before it is worked on
+        float q_next[RPT], k_next[RPT], g_next[RPT], b_next, v_next;
+        auto fetch = [&](int token) {
             const float* t0 = staged + token * TOKEN;
-            const float* qs = t0 + quarter * RPT;
-            const float* ks = t0 + DP + quarter * RPT;
-            const float* gs = t0 + 2 * DP + quarter * RPT;
-            const float b = t0[3 * DP];
-            const float v = t0[3 * DP + 4 + threadIdx.x / 4];
+#pragma unroll
+            for (int t = 0; t < RPT; ++t) {
+                q_next[t] = t0[part * RPT + t];
+                k_next[t] = t0[DP + part * RPT + t];
+                g_next[t] = t0[2 * DP + part * RPT + t];
+            }
+            b_next = t0[3 * DP];
+            v_next = t0[3 * DP + 4 + local];
+        };
+        fetch(0);
+        for (int token = 0; token < tokens; ++token) {
+            float q_now[RPT], k_now[RPT];
+            const float b = b_next, v = v_next;
             float seen = 0.0f;
 #pragma unroll
             for (int t = 0; t < RPT; ++t) {
-                S[t] *= gs[t];
-                seen = fmaf(S[t], ks[t], seen);
+                q_now[t] = q_next[t];
+                k_now[t] = k_next[t];
+                S[t] *= g_next[t];
+                seen = fmaf(S[t], k_now[t], seen);
             }
-            seen += __shfl_xor(seen, 1, 64);
-            seen += __shfl_xor(seen, 2, 64);
+            fetch(token + 1 < DELTA_CHUNK ? token + 1 : token);      // (behind the chunk's last token: read again, not used)
+            seen = delta_row_sum(seen);
             const float u = b * (v - seen);
             float read = 0.0f;
 #pragma unroll
             for (int t = 0; t < RPT; ++t) {
-                S[t] = fmaf(ks[t], u, S[t]);
-                read = fmaf(S[t], qs[t], read);
+                S[t] = fmaf(k_now[t], u, S[t]);
+                read = fmaf(S[t], q_now[t], read);
             }
-            read += __shfl_xor(read, 1, 64);
-            read += __shfl_xor(read, 2, 64);
-            if (live && quarter == 0) out[((size_t)first + base + token) * heads * vdim + head * vdim + column] = read;
+            read = delta_row_sum(read);
+            if (part == 0) results[token * DELTA_COLUMNS + local] = read;
+        }
+        __syncthreads();
+        // the chunk's read-outs leave together: a token's 16 columns side by side
+        {
+            const int token = threadIdx.x / DELTA_COLUMNS, c = threadIdx.x % DELTA_COLUMNS;
+            if (token < tokens && block * DELTA_COLUMNS + c < vdim)
+                out[((size_t)first + base + token) * heads * vdim + head * vdim + block * DELTA_COLUMNS + c] = results[threadIdx.x];
         }
         __syncthreads();
         if (more) put(base + DELTA_CHUNK);
@@ -279,7 +318,7 @@ __global__ __launch_bounds__(256) void gated_delta_rule_kernel(
     if (live) {
 #pragma unroll
         for (int t = 0; t < RPT; ++t) {
-            const int i = quarter * RPT + t;
+            const int i = part * RPT + t;
             if (i < dim) mine[i] = S[t];
         }
     }
@@ -297,11 +336,11 @@ extern "C" int fw_gated_delta_rule(const float* records, float* state, float* ou
     hipStream_t s = (hipStream_t)stream;
 #define FW_DELTA_LAUNCH(RPT) \
     gated_delta_rule_kernel<RPT><<<grid, 256, 0, s>>>(records, state, out, seg_row0, seg_slot, heads, dim, vdim)
-    if (dim <= 16) FW_DELTA_LAUNCH(4);
-    else if (dim <= 32) FW_DELTA_LAUNCH(8);
-    else if (dim <= 64) FW_DELTA_LAUNCH(16);
-    else if (dim <= 128) FW_DELTA_LAUNCH(32);
-    else FW_DELTA_LAUNCH(64);
+    if (dim <= 16) FW_DELTA_LAUNCH(1);
+    else if (dim <= 32) FW_DELTA_LAUNCH(2);
+    else if (dim <= 64) FW_DELTA_LAUNCH(4);
+    else if (dim <= 128) FW_DELTA_LAUNCH(8);
+    else FW_DELTA_LAUNCH(16);
 #undef FW_DELTA_LAUNCH
     FW_LAUNCH_CHECK("gated_delta_rule");
     return 0;

@@ -22,16 +22,20 @@ __global__ __launch_bounds__(256) void norm_scale_add_kernel(
     __shared__ float scratch[16];
     const size_t row0 = (size_t)blockIdx.x * hidden;
     const bool held_all = hidden <= 256 * NORM_ADD_HELD;
-    float held[NORM_ADD_HELD];
+    float held[NORM_ADD_HELD], was[NORM_ADD_HELD], scale[NORM_ADD_HELD];
     float sum = 0.0f;
     if (held_all) {
+        // everything the row needs is asked for at once: the old x and the weight travel with a and b
 #pragma unroll
         for (int u = 0; u < NORM_ADD_HELD; ++u) {
             const int i = threadIdx.x + 256 * u;
             float y = 0.0f;
+            was[u] = scale[u] = 0.0f;
             if (i < hidden) {
                 y = scale_a * a[row0 + i];
                 if (b) y = fmaf(scale_b, b[row0 + i], y);
+                was[u] = x[row0 + i];
+                scale[u] = weight[i];
             }
             held[u] = y;
             sum = fmaf(y, y, sum);
@@ -51,7 +55,7 @@ __global__ __launch_bounds__(256) void norm_scale_add_kernel(
         for (int u = 0; u < NORM_ADD_HELD; ++u) {
             const int i = threadIdx.x + 256 * u;
             if (i < hidden) {
-                const float updated = x[row0 + i] + mult * (held[u] * inv * (weight[i] + one));
+                const float updated = was[u] + mult * (held[u] * inv * (scale[u] + one));
                 x[row0 + i] = updated;
                 if (rounded) store_from_float(rounded, row0 + i, updated);
             }
