@@ -105,6 +105,16 @@ def koketar_run(torch, args) -> dict:
     import numpy as np
     results = {}
     steps = min(args.steps, 64)
+    if args.only:       # one phase of Koketar at width 2,048 alone, no JSON (for profiling)
+        config = koketar_configs(KOKETAR_SIZES["w2048"])[0]
+        model = Model.random(config, seed=0, dtype="bfloat16")
+        if args.only == "prefill":
+            seconds, _ = prefill_run(torch, model, config, repeats=3)
+            log(f"{PROMPT / seconds:.1f} tokens/s")
+        else:
+            seconds, _, _ = decode_run(torch, model, config, args.batch, steps, min(args.warmup, 8))
+            log(f"{args.batch * steps / seconds:.1f} tokens/s")
+        return None
     for size_name, size in KOKETAR_SIZES.items():
         for family, config in zip(("koketar", "lfm2"), koketar_configs(size)):
             log(f"{family} {size_name}: random bfloat16 weights")
@@ -459,7 +469,9 @@ def main() -> int:
     from flyweight_amd.config import config_from_dict
 
     if args.workload == "koketar":
-        print(json.dumps(koketar_run(torch, args)), flush=True)
+        record = koketar_run(torch, args)
+        if record is not None:
+            print(json.dumps(record), flush=True)
         return 0
     if args.workload != "headline":
         print(json.dumps(serving_run(torch, args.workload, args.requests or WORKLOADS[args.workload]["requests"])), flush=True)

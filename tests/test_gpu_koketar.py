@@ -220,3 +220,27 @@ def test_trace_replay(models, tmp_path):
     assert_close(read(1), full_a[[68]], "float32", "step 1")
     assert_close(read(2), np.stack([full_a[69], full_b[8]]), "float32", "step 2")
     assert_close(read(3), full_b[[8]], "float32", "step 3")
+
+
+def test_command_line(models, capsys, tmp_path):
+    """generate prints the plain model's greedy tokens; inspect names the architecture and its
+    tensors; random-weights writes a folder from a configuration that gives the low-rank widths."""
+    import json
+    from flyweight_amd.cli import main
+    from flyweight_amd.config import load_config
+    loaded = models("Y", "float32")
+    prompt = random_tokens(loaded.config["vocab"], 13, seed=40)
+    expected = plain.greedy(loaded.config, loaded.weights, prompt, 5)
+    assert main(["generate", loaded.folder, "--tokens", ",".join(map(str, prompt)), "--max-tokens", "5", "--temperature", "0",
+                 "--dtype", "float32", "--ignore-eos", "--context", "128"]) == 0
+    assert [int(t) for t in capsys.readouterr().out.split()] == expected
+    assert main(["inspect", loaded.folder]) == 0
+    shown = json.loads(capsys.readouterr().out)
+    assert shown["architecture"] == "Koketar" and set(shown["tensors"]) == set(plain.tensor_shapes(loaded.config))
+    described = load_config(loaded.folder).to_dict()            # with the ranks the tensors showed
+    (tmp_path / "config.json").write_text(json.dumps(described))
+    assert main(["random-weights", "--config", str(tmp_path / "config.json"), "--seed", "3", "--out", str(tmp_path / "drawn")]) == 0
+    capsys.readouterr()
+    assert main(["generate", str(tmp_path / "drawn"), "--tokens", "1,2,3", "--max-tokens", "4", "--temperature", "0",
+                 "--ignore-eos", "--context", "128"]) == 0
+    assert len(capsys.readouterr().out.split()) == 4
