@@ -43,7 +43,9 @@ __device__ __forceinline__ uint32_t pack_bf16_pair(float lo, float hi) {
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
 }
 
-// State of one wave: 16 columns, HD channels (HD a multiple of 32; channels >= head_dim are zero).
+// State of one wave: 16 columns, HD channels (HD a multiple of 32 that holds both a key's head_dim
+// channels and a value's v_dim channels, which may differ; query channels >= head_dim are zero, output
+// channels >= v_dim are computed from the last real one and never stored).
 template <int HD>
 struct Columns {
     bf16x8 q[HD / 32];          // this lane's part of Q^T: column lane % 16, d = 32 c + 8 (lane / 16) ..
@@ -71,7 +73,7 @@ struct Columns {
 // scores (the scale is positive) and kept scaled.
 template <int HD, int NH, bool CLEAN_V, bool K_PADDED, bool EARLY_V = false>
 __device__ __forceinline__ void attend_page(Columns<HD> (&c)[NH], const uint16_t* __restrict__ k_page,
-                                            const uint16_t* __restrict__ v_page, int head_dim, float scale_log2,
+                                            const uint16_t* __restrict__ v_page, int head_dim, int v_dim, float scale_log2,
                                             int lo, int hi, int last_written, int k_stride, int v_stride) {
     const int lane = threadIdx.x & 63;
     const int i16 = lane & 15, g = lane >> 4;
@@ -98,7 +100,7 @@ __device__ __forceinline__ void attend_page(Columns<HD> (&c)[NH], const uint16_t
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
             for (int t = 0; t < HD / 16; ++t) {
-                const int channel = t * 16 + i16 < head_dim ? t * 16 + i16 : head_dim - 1;
+                const int channel = t * 16 + i16 < v_dim ? t * 16 + i16 : v_dim - 1;
                 const uint16_t* value = v_page + (size_t)channel * v_stride + kb * 32 + g * 4;
                 early_a[kb][t] = *reinterpret_cast<const u32x2*>(value);
                 early_b[kb][t] = *reinterpret_cast<const u32x2*>(value + 16);
@@ -204,7 +206,7 @@ __device__ __forceinline__ void attend_page(Columns<HD> (&c)[NH], const uint16_t
         // components stale).
 #pragma unroll
         for (int t = 0; t < HD / 16; ++t) {
-            const int channel = t * 16 + i16 < head_dim ? t * 16 + i16 : head_dim - 1;
+            const int channel = t * 16 + i16 < v_dim ? t * 16 + i16 : v_dim - 1;
             const uint16_t* value = v_page + (size_t)channel * v_stride;
             u32x2 va, vb;
             if (EARLY_V) {
@@ -262,12 +264,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((HD <= 64 &
     const uint16_t* __restrict__ q, uint16_t* __restrict__ out, const uint16_t* __restrict__ k_pages,
     const uint16_t* __restrict__ v_pages, const int32_t* __restrict__ block_table, int table_stride,
     const int32_t* __restrict__ tile_seg, const int32_t* __restrict__ tile_row0, const int32_t* __restrict__ seg_row0,
-    const int32_t* __restrict__ row_pos, int num_heads, int num_kv_heads, int head_dim, float scale_log2, int window) {
+    const int32_t* __restrict__ row_pos, int num_heads, int num_kv_heads, int head_dim, int v_dim, float scale_log2, int window) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     // a key's row in LDS holds HD channels, those past head_dim zero: every lane loads its operand
     constexpr int k_stride = HD + KV_PAD;
     const int v_stride = PAGE + KV_PAD;
-    const int k_elems = PAGE * k_stride, v_elems = head_dim * v_stride;
+    const int k_elems = PAGE * k_stride, v_elems = v_dim * v_stride;
     uint16_t* lds = reinterpret_cast<uint16_t*>(lds_raw);      // [buffer][K tile | V tile]
     if (head_dim < HD) {
         const int runs_per_row = (HD - head_dim) / 8;          // head_dim is a multiple of 16
@@ -305,31 +307,33 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((HD <= 64 &
         load_query<HD>(c[h], q + ((size_t)my_row * num_heads + head) * head_dim, head_dim, valid && head_there);
     }
     const int32_t* table = block_table + (size_t)seg * table_stride;
-    const size_t page_elems = (size_t)PAGE * head_dim;
+    const size_t k_page_elems = (size_t)PAGE * head_dim, v_page_elems = (size_t)PAGE * v_dim;
 
-    // the copy: a page's K is 64 rows of head_dim, its V head_dim rows of 64; runs of 16 bytes.
+    // the copy: a page's K is 64 rows of head_dim, its V v_dim rows of 64; runs of 16 bytes.
     // Loads are unconditional (a run or a page past the end is read from a valid place again and
     // never used) and the barriers order LDS traffic only, so that the pages requested stay in
     // flight while the page before them is worked on.
-    const int k_runs = PAGE * head_dim / 8;                                      // as many for V
+    const int k_runs = PAGE * head_dim / 8, v_runs = PAGE * v_dim / 8;
     constexpr int MAX_RUNS = HD * PAGE / 8 / 256;                                // per thread, per operand
     const int first_block = tile_first / PAGE, last_block = pos_hi / PAGE;
     u32x4 hold_k0[MAX_RUNS], hold_v0[MAX_RUNS], hold_k1[MAX_RUNS], hold_v1[MAX_RUNS];
     // what a thread copies of every page: fixed offsets, so that a page's address is a scalar
     // base plus these (no vector arithmetic per page; the registers that receive a page are
     // otherwise borrowed for it, and giving them back means waiting for loads still in flight)
-    uint32_t run_offset[MAX_RUNS];
+    uint32_t run_offset[MAX_RUNS], run_offset_v[MAX_RUNS];
 #pragma unroll
-    for (int u = 0; u < MAX_RUNS; ++u) run_offset[u] = (uint32_t)(tid + u * 256 < k_runs ? tid + u * 256 : 0) * 8u;
+    for (int u = 0; u < MAX_RUNS; ++u) {
+        run_offset[u] = (uint32_t)(tid + u * 256 < k_runs ? tid + u * 256 : 0) * 8u;
+        run_offset_v[u] = (uint32_t)(tid + u * 256 < v_runs ? tid + u * 256 : 0) * 8u;
+    }
     auto fetch = [&](u32x4 (&hold_k)[MAX_RUNS], u32x4 (&hold_v)[MAX_RUNS], int block) {
         const int page = __builtin_amdgcn_readfirstlane(table[block < last_block ? block : last_block]);
-        const size_t at = ((size_t)page * num_kv_heads + kvh) * page_elems;
-        const uint16_t* k_from = k_pages + at;
-        const uint16_t* v_from = v_pages + at;
+        const uint16_t* k_from = k_pages + ((size_t)page * num_kv_heads + kvh) * k_page_elems;
+        const uint16_t* v_from = v_pages + ((size_t)page * num_kv_heads + kvh) * v_page_elems;
 #pragma unroll
         for (int u = 0; u < MAX_RUNS; ++u) {
             hold_k[u] = *reinterpret_cast<const u32x4*>(k_from + run_offset[u]);
-            hold_v[u] = *reinterpret_cast<const u32x4*>(v_from + run_offset[u]);
+            hold_v[u] = *reinterpret_cast<const u32x4*>(v_from + run_offset_v[u]);
         }
     };
     // The values of keys past the last one written (only in the tile's last page) are zeroed on
@@ -342,8 +346,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((HD <= 64 &
 #pragma unroll
         for (int u = 0; u < MAX_RUNS; ++u) {
             const int run = tid + u * 256;
-            if (run < k_runs) {
-                *reinterpret_cast<u32x4*>(kt + (run / k_per_row) * k_stride + (run % k_per_row) * 8) = hold_k[u];
+            if (run < k_runs) *reinterpret_cast<u32x4*>(kt + (run / k_per_row) * k_stride + (run % k_per_row) * 8) = hold_k[u];
+            if (run < v_runs) {
                 u32x4 v = hold_v[u];
                 if (last_written < PAGE - 1) {
                     const int key0 = (run % 8) * 8;             // this run: keys key0 .. key0 + 7 of one channel
@@ -363,7 +367,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((HD <= 64 &
             const uint16_t* kt = lds + (size_t)buffer * (k_elems + v_elems);
             // a lane without a row computes along with the bounds of the tile's first row (nothing of
             // it is stored): a page that is whole for the rows is then whole for the wave
-            attend_page<HD, NH, false, true>(c, kt, kt + k_elems, head_dim, scale_log2, my_first - base, my_pos - base, pos_hi - base,
+            attend_page<HD, NH, false, true>(c, kt, kt + k_elems, head_dim, v_dim, scale_log2, my_first - base, my_pos - base, pos_hi - base,
                             k_stride, v_stride);
         }
     };
@@ -392,10 +396,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((HD <= 64 &
         const float l = fw_quad_sum(c[h].l);
         if (!valid || first_in_group + h >= group) continue;
         const float inv = 1.0f / l;
-        uint16_t* dest = out + ((size_t)my_row * num_heads + kvh * group + first_in_group + h) * head_dim;
+        uint16_t* dest = out + ((size_t)my_row * num_heads + kvh * group + first_in_group + h) * v_dim;
 #pragma unroll
         for (int t = 0; t < HD / 16; ++t) {
-            if (t * 16 >= head_dim) break;
+            if (t * 16 >= v_dim) break;
             u32x2 packed = {pack_bf16(c[h].o[t][0] * inv, c[h].o[t][1] * inv), pack_bf16(c[h].o[t][2] * inv, c[h].o[t][3] * inv)};
             *reinterpret_cast<u32x2*>(dest + t * 16 + g * 4) = packed;
         }
@@ -406,12 +410,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((HD <= 64 &
 #define DECODE_WORKGROUPS 512        // two per compute unit: beyond, longer splits serve better than more of them
 // grid (rows, kv heads * head tiles, splits); four waves, each takes one page of the split's
 // SPLIT_PAGES, and their results are merged in LDS in the order of the keys. Columns are the
-// query heads of the kv group (16 per head tile). partial [rows][heads][max_splits][head_dim + 4]:
+// query heads of the kv group (16 per head tile). partial [rows][heads][max_splits][v_dim + 4]:
 // unnormalised output, then maximum and sum; a split with nothing to do writes nothing and takes
 // no ticket. The last workgroup of a (row, kv head, head tile) to arrive merges what the others
 // left; the only workgroup of a short row writes the result at once.
 // What the fused variant does in front of the attention: the step's raw projections (float32
-// [rows][(heads + 2 kv heads) * head_dim]: queries, keys, values) get their per-head RMS norm and
+// [rows][(heads + kv heads) * head_dim + kv heads * v_dim]: queries, keys, values) get their per-head RMS norm and
 // rotation here, as qk_norm_rope_kv_write does in a kernel of its own (the same arithmetic in the
 // same order), so that a decode step needs no such kernel. Every workgroup norms and rotates the
 // query heads it works on; the workgroup whose pages include the row's own position also norms and
@@ -471,7 +475,7 @@ __global__ __launch_bounds__(64 * SPLIT_PAGES) __attribute__((amdgpu_waves_per_e
     const uint16_t* __restrict__ q, uint16_t* __restrict__ out, float* partial, int* tickets,
     uint16_t* k_pages, uint16_t* v_pages, const int32_t* __restrict__ block_table, int table_stride,
     const int32_t* __restrict__ row_seg, const int32_t* __restrict__ row_pos, int num_heads, int num_kv_heads,
-    int head_dim, float scale_log2, int window, int max_splits, const int32_t* __restrict__ decode_work, const FusedProjections fused) {
+    int head_dim, int v_dim, float scale_log2, int window, int max_splits, const int32_t* __restrict__ decode_work, const FusedProjections fused) {
     __shared__ f32x4 shared_o[SPLIT_PAGES][HD / 16][64];
     __shared__ float shared_m[SPLIT_PAGES][16], shared_l[SPLIT_PAGES][16];
     __shared__ int ticket_shared;
@@ -508,7 +512,7 @@ __global__ __launch_bounds__(64 * SPLIT_PAGES) __attribute__((amdgpu_waves_per_e
     Columns<HD> columns_of_wave[1];
     Columns<HD>& c = columns_of_wave[0];
     if (FUSED) {
-        const int width = (num_heads + 2 * num_kv_heads) * head_dim;
+        const int width = (num_heads + num_kv_heads) * head_dim + num_kv_heads * v_dim;
         const float* projections = fused.qkv + (size_t)row * width;
         const int half = fused.rotary_dim / 2;
         const float* cos_row = fused.cos_table + (size_t)row * half;
@@ -532,9 +536,9 @@ __global__ __launch_bounds__(64 * SPLIT_PAGES) __attribute__((amdgpu_waves_per_e
                                    fused.rotary_dim, head_dim, fused_scratch[wave],
                                    [&](int d, float value) { dest[d] = float_to_bf16_bits(value); });
             } else {
-                const float* value = projections + (size_t)(num_heads + num_kv_heads + kvh) * head_dim;
-                uint16_t* dest = v_pages + ((size_t)own_page * num_kv_heads + kvh) * head_dim * PAGE + slot;
-                for (int d = lane; d < head_dim; d += 64) dest[(size_t)d * PAGE] = float_to_bf16_bits(value[d]);
+                const float* value = projections + (size_t)(num_heads + num_kv_heads) * head_dim + (size_t)kvh * v_dim;
+                uint16_t* dest = v_pages + ((size_t)own_page * num_kv_heads + kvh) * v_dim * PAGE + slot;
+                for (int d = lane; d < v_dim; d += 64) dest[(size_t)d * PAGE] = float_to_bf16_bits(value[d]);
             }
         }
         // the page is read below by this workgroup's own waves: its stores have to be done first
@@ -548,10 +552,10 @@ __global__ __launch_bounds__(64 * SPLIT_PAGES) __attribute__((amdgpu_waves_per_e
         const int block = first_block + round * SPLIT_PAGES + wave;
         if (block > last_block) break;
         const int page = block_table[(size_t)segment * table_stride + block];
-        const size_t at = ((size_t)page * num_kv_heads + kvh) * PAGE * head_dim;
+        const size_t at = ((size_t)page * num_kv_heads + kvh) * PAGE;
         const int base = block * PAGE;
         // a lane without a head computes along (q = 0, nothing of it is stored)
-        attend_page<HD, 1, true, false, (HD <= 128)>(columns_of_wave, k_pages + at, v_pages + at, head_dim, scale_log2, first - base, pos - base, pos - base,
+        attend_page<HD, 1, true, false, (HD <= 128)>(columns_of_wave, k_pages + at * head_dim, v_pages + at * v_dim, head_dim, v_dim, scale_log2, first - base, pos - base, pos - base,
                         head_dim, PAGE);
     }
     const float l = fw_quad_sum(c.l);
@@ -564,7 +568,7 @@ __global__ __launch_bounds__(64 * SPLIT_PAGES) __attribute__((amdgpu_waves_per_e
     __syncthreads();
     // how many workgroups work on this row: those whose first page holds a visible key
     const int row_splits = (last_block - first / PAGE + 1 + pages_per_split - 1) / pages_per_split;
-    const int stride = PART_STRIDE(head_dim);
+    const int stride = PART_STRIDE(v_dim);
     if (wave == 0 && valid) {
         float m = NEG_BIG;
 #pragma unroll
@@ -576,10 +580,10 @@ __global__ __launch_bounds__(64 * SPLIT_PAGES) __attribute__((amdgpu_waves_per_e
             total += weight[w] * shared_l[w][col];
         }
         float* dest = partial + (((size_t)row * num_heads + head) * max_splits + split) * stride;
-        uint16_t* final_dest = out + ((size_t)row * num_heads + head) * head_dim;
+        uint16_t* final_dest = out + ((size_t)row * num_heads + head) * v_dim;
 #pragma unroll
         for (int t = 0; t < HD / 16; ++t) {
-            if (t * 16 >= head_dim) break;
+            if (t * 16 >= v_dim) break;
             f32x4 sum = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int w = 0; w < SPLIT_PAGES; ++w) sum += weight[w] * shared_o[w][t][lane];
@@ -596,8 +600,8 @@ __global__ __launch_bounds__(64 * SPLIT_PAGES) __attribute__((amdgpu_waves_per_e
             }
         }
         if (g == 0 && row_splits > 1) {
-            __hip_atomic_store(dest + head_dim, m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_store(dest + head_dim + 1, total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(dest + v_dim, m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(dest + v_dim + 1, total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     }
     if (row_splits == 1) return;
@@ -612,8 +616,8 @@ __global__ __launch_bounds__(64 * SPLIT_PAGES) __attribute__((amdgpu_waves_per_e
     if (ticket_shared != row_splits - 1) return;
     if (threadIdx.x == 0) __hip_atomic_store(ticket, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     const int columns = group - head_tile * 16 < 16 ? group - head_tile * 16 : 16;
-    for (int item = threadIdx.x; item < columns * head_dim; item += 64 * SPLIT_PAGES) {
-        const int merged_head = kvh * group + head_tile * 16 + item / head_dim, d = item % head_dim;
+    for (int item = threadIdx.x; item < columns * v_dim; item += 64 * SPLIT_PAGES) {
+        const int merged_head = kvh * group + head_tile * 16 + item / v_dim, d = item % v_dim;
         const float* source = partial + ((size_t)row * num_heads + merged_head) * max_splits * stride;
         // Sixteen parts are requested at a time (past the last one: the last one again, not used),
         // maximum, weight and value together: one round trip for up to sixteen parts. The running
@@ -628,8 +632,8 @@ __global__ __launch_bounds__(64 * SPLIT_PAGES) __attribute__((amdgpu_waves_per_e
             float ms[AT_ONCE], ls[AT_ONCE], vs[AT_ONCE];
 #pragma unroll
             for (int u = 0; u < AT_ONCE; ++u) {
-                ms[u] = part_at(sp0 + u, head_dim);
-                ls[u] = part_at(sp0 + u, head_dim + 1);
+                ms[u] = part_at(sp0 + u, v_dim);
+                ls[u] = part_at(sp0 + u, v_dim + 1);
                 vs[u] = part_at(sp0 + u, d);
             }
             float highest = m;
@@ -646,17 +650,18 @@ __global__ __launch_bounds__(64 * SPLIT_PAGES) __attribute__((amdgpu_waves_per_e
                 acc += weight * vs[u];
             }
         }
-        out[((size_t)row * num_heads + merged_head) * head_dim + d] = float_to_bf16_bits(acc / total);
+        out[((size_t)row * num_heads + merged_head) * v_dim + d] = float_to_bf16_bits(acc / total);
     }
 }
 
 static const float LOG2E = 1.4426950408889634f;
 
-static int check_common(const char* name, int rows, int num_heads, int num_kv_heads, int head_dim, int page_size,
+static int check_common(const char* name, int rows, int num_heads, int num_kv_heads, int head_dim, int v_dim, int page_size,
                         int window, int num_pages, int table_stride) {
     FW_REQUIRE(rows >= 0 && num_heads > 0 && num_kv_heads > 0 && num_heads % num_kv_heads == 0,
                "%s: heads %d must be a positive multiple of kv heads %d", name, num_heads, num_kv_heads);
     FW_REQUIRE(head_dim >= 16 && head_dim <= 256 && head_dim % 16 == 0, "%s: head_dim %d must be a multiple of 16 in 16..256", name, head_dim);
+    FW_REQUIRE(v_dim >= 16 && v_dim <= 256 && v_dim % 16 == 0, "%s: the values' size %d must be a multiple of 16 in 16..256", name, v_dim);
     FW_REQUIRE(page_size == PAGE, "%s: page size must be %d, got %d", name, PAGE, page_size);
     FW_REQUIRE(window >= 0, "%s: window must be 0 (all keys) or positive, got %d", name, window);
     FW_REQUIRE(num_pages > 0 && table_stride > 0, "%s: empty cache (pages=%d, table stride=%d)", name, num_pages, table_stride);
@@ -683,11 +688,12 @@ extern "C" int fw_attention_prefill(const void* q, void* out, const void* k_page
                                     const int32_t* block_table, int table_stride, const int32_t* tile_seg,
                                     const int32_t* tile_row0, int tiles, const int32_t* seg_row0,
                                     const int32_t* row_pos, int rows, int num_heads, int num_kv_heads, int head_dim,
-                                    float scale, int window, int page_size, int num_pages, int heads_together,
+                                    int v_dim, float scale, int window, int page_size, int num_pages, int heads_together,
                                     void* stream) {
-    if (check_common("attention_prefill", rows, num_heads, num_kv_heads, head_dim, page_size, window, num_pages, table_stride)) return -1;
+    if (check_common("attention_prefill", rows, num_heads, num_kv_heads, head_dim, v_dim, page_size, window, num_pages, table_stride)) return -1;
+    const int widest = head_dim > v_dim ? head_dim : v_dim;      // the template holds both
     FW_REQUIRE(tiles >= 0 && tiles <= rows && num_heads <= 65535, "attention_prefill: %d tiles for %d rows", tiles, rows);
-    const int most_together = head_dim <= 64 ? 4 : 1;
+    const int most_together = widest <= 64 ? 4 : 1;
     FW_REQUIRE(heads_together == 0 || heads_together == 1 || (heads_together == 4 && most_together == 4),
                "attention_prefill: %d heads together with head_dim %d (1, or 4 up to head_dim 64)", heads_together, head_dim);
     if (rows == 0 || tiles == 0) return 0;
@@ -699,7 +705,7 @@ extern "C" int fw_attention_prefill(const void* q, void* out, const void* k_page
     dim3 grid((unsigned)blocks);
 #define LAUNCH(HD, NH)                                                                                             \
     {                                                                                                              \
-        const int lds_bytes = 2 * (PAGE * (HD + KV_PAD) + head_dim * (PAGE + KV_PAD)) * 2;                         \
+        const int lds_bytes = 2 * (PAGE * (HD + KV_PAD) + v_dim * (PAGE + KV_PAD)) * 2;                            \
         static int configured = 0;                                                                                 \
         if (lds_bytes > configured) {                                                                              \
             hipError_t status = hipFuncSetAttribute((const void*)attention_prefill_kernel<HD, NH>,                 \
@@ -709,14 +715,14 @@ extern "C" int fw_attention_prefill(const void* q, void* out, const void* k_page
         }                                                                                                          \
         attention_prefill_kernel<HD, NH><<<grid, 256, lds_bytes, (hipStream_t)stream>>>(                            \
             (const uint16_t*)q, (uint16_t*)out, (const uint16_t*)k_pages, (const uint16_t*)v_pages, block_table,    \
-            table_stride, tile_seg, tile_row0, seg_row0, row_pos, num_heads, num_kv_heads, head_dim, scale * LOG2E, \
-            window);                                                                                               \
+            table_stride, tile_seg, tile_row0, seg_row0, row_pos, num_heads, num_kv_heads, head_dim, v_dim,        \
+            scale * LOG2E, window);                                                                                \
     }
-    if (head_dim <= 32) {
+    if (widest <= 32) {
         if (heads_together == 4) LAUNCH(32, 4) else LAUNCH(32, 1)
-    } else if (head_dim <= 64) {
+    } else if (widest <= 64) {
         if (heads_together == 4) LAUNCH(64, 4) else LAUNCH(64, 1)
-    } else if (head_dim <= 128) {
+    } else if (widest <= 128) {
         LAUNCH(128, 1)
     } else {
         LAUNCH(256, 1)
@@ -727,8 +733,8 @@ extern "C" int fw_attention_prefill(const void* q, void* out, const void* k_page
 }
 
 static int decode_check(int max_splits, int max_context, int* tickets, int tickets_len, int table_stride, int rows, int num_heads,
-                        int num_kv_heads, int head_dim, int window, int page_size, int num_pages) {
-    if (check_common("attention_decode", rows, num_heads, num_kv_heads, head_dim, page_size, window, num_pages, table_stride)) return -1;
+                        int num_kv_heads, int head_dim, int v_dim, int window, int page_size, int num_pages) {
+    if (check_common("attention_decode", rows, num_heads, num_kv_heads, head_dim, v_dim, page_size, window, num_pages, table_stride)) return -1;
     FW_REQUIRE(max_splits >= 1 && max_splits <= 65535, "attention_decode: max_splits %d outside 1..65535", max_splits);
     FW_REQUIRE(max_context >= 1, "attention_decode: max_context must be positive");
     int blocks = (max_context + PAGE - 1) / PAGE;
@@ -746,7 +752,7 @@ static int decode_check(int max_splits, int max_context, int* tickets, int ticke
 
 static int decode_launch(const void* q, void* out, float* partial, int max_splits, const int32_t* decode_work, int* tickets, void* k_pages, void* v_pages,
                          const int32_t* block_table, int table_stride, const int32_t* row_seg, const int32_t* row_pos, int rows,
-                         int num_heads, int num_kv_heads, int head_dim, float scale, int window, const FusedProjections& fused,
+                         int num_heads, int num_kv_heads, int head_dim, int v_dim, float scale, int window, const FusedProjections& fused,
                          void* stream) {
     if (rows == 0) return 0;
     const int head_tiles = (num_heads / num_kv_heads + 15) / 16;
@@ -756,12 +762,12 @@ static int decode_launch(const void* q, void* out, float* partial, int max_split
     if (fused.qkv)                                                                                                            \
         attention_decode_split_kernel<HD, true><<<grid, 64 * SPLIT_PAGES, 0, (hipStream_t)stream>>>(                          \
             (const uint16_t*)q, (uint16_t*)out, partial, tickets, (uint16_t*)k_pages, (uint16_t*)v_pages, block_table,        \
-            table_stride, row_seg, row_pos, num_heads, num_kv_heads, head_dim, scale * LOG2E, window, max_splits, decode_work, fused); \
+            table_stride, row_seg, row_pos, num_heads, num_kv_heads, head_dim, v_dim, scale * LOG2E, window, max_splits, decode_work, fused); \
     else                                                                                                                      \
         attention_decode_split_kernel<HD, false><<<grid, 64 * SPLIT_PAGES, 0, (hipStream_t)stream>>>(                         \
             (const uint16_t*)q, (uint16_t*)out, partial, tickets, (uint16_t*)k_pages, (uint16_t*)v_pages, block_table,        \
-            table_stride, row_seg, row_pos, num_heads, num_kv_heads, head_dim, scale * LOG2E, window, max_splits, decode_work, fused)
-    FW_BY_HEAD_DIM(head_dim, CALL);
+            table_stride, row_seg, row_pos, num_heads, num_kv_heads, head_dim, v_dim, scale * LOG2E, window, max_splits, decode_work, fused)
+    FW_BY_HEAD_DIM((head_dim > v_dim ? head_dim : v_dim), CALL);
 #undef CALL
     FW_LAUNCH_CHECK("attention_decode");
     return 0;
@@ -779,12 +785,12 @@ extern "C" int fw_attention_decode(const void* q, void* out, float* partial, int
                                    const int32_t* decode_work, int* tickets, int tickets_len, const void* k_pages,
                                    const void* v_pages, const int32_t* block_table, int table_stride,
                                    const int32_t* row_seg, const int32_t* row_pos, int rows, int num_heads,
-                                   int num_kv_heads, int head_dim, float scale, int window, int page_size,
+                                   int num_kv_heads, int head_dim, int v_dim, float scale, int window, int page_size,
                                    int num_pages, void* stream) {
-    if (decode_check(max_splits, max_context, tickets, tickets_len, table_stride, rows, num_heads, num_kv_heads, head_dim, window,
+    if (decode_check(max_splits, max_context, tickets, tickets_len, table_stride, rows, num_heads, num_kv_heads, head_dim, v_dim, window,
                      page_size, num_pages)) return -1;
     return decode_launch(q, out, partial, max_splits, decode_work, tickets, const_cast<void*>(k_pages), const_cast<void*>(v_pages), block_table,
-                         table_stride, row_seg, row_pos, rows, num_heads, num_kv_heads, head_dim, scale, window, FusedProjections{}, stream);
+                         table_stride, row_seg, row_pos, rows, num_heads, num_kv_heads, head_dim, v_dim, scale, window, FusedProjections{}, stream);
 }
 
 // fw_attention_decode with the work of fw_qk_norm_rope_kv_write in front of it, in the same kernel:
@@ -797,9 +803,9 @@ extern "C" int fw_attention_decode_fused(const float* qkv, const float* q_norm_w
                                          float* partial, int max_splits, int max_context, const int32_t* decode_work, int* tickets, int tickets_len,
                                          void* k_pages, void* v_pages, const int32_t* block_table, int table_stride,
                                          const int32_t* row_seg, const int32_t* row_pos, int rows, int num_heads,
-                                         int num_kv_heads, int head_dim, float scale, int window, int page_size, int num_pages,
+                                         int num_kv_heads, int head_dim, int v_dim, float scale, int window, int page_size, int num_pages,
                                          void* stream) {
-    if (decode_check(max_splits, max_context, tickets, tickets_len, table_stride, rows, num_heads, num_kv_heads, head_dim, window,
+    if (decode_check(max_splits, max_context, tickets, tickets_len, table_stride, rows, num_heads, num_kv_heads, head_dim, v_dim, window,
                      page_size, num_pages)) return -1;
     FW_REQUIRE(qkv != nullptr, "attention_decode_fused: the projections are missing");
     FW_REQUIRE(rotary_dim >= 0 && rotary_dim <= head_dim && rotary_dim % 2 == 0, "attention_decode_fused: rotary_dim %d with head_dim %d",
@@ -810,5 +816,5 @@ extern "C" int fw_attention_decode_fused(const float* qkv, const float* q_norm_w
     fused.qkv = qkv; fused.q_norm_weight = q_norm_weight; fused.k_norm_weight = k_norm_weight; fused.eps = eps;
     fused.cos_table = cos_table; fused.sin_table = sin_table; fused.rotary_dim = rotary_dim; fused.write_kv = write_kv;
     return decode_launch(nullptr, out, partial, max_splits, decode_work, tickets, k_pages, v_pages, block_table, table_stride, row_seg, row_pos,
-                         rows, num_heads, num_kv_heads, head_dim, scale, window, fused, stream);
+                         rows, num_heads, num_kv_heads, head_dim, v_dim, scale, window, fused, stream);
 }

@@ -156,6 +156,19 @@ __device__ __forceinline__ float block_sum(float v, float* scratch /* >= 16 floa
     return total;
 }
 
+// A gated unit behind a product that holds gate and up of one feature: silu(g) * u (limit <= 0), or
+// with clamped halves g' = min(g, limit), u' = clamp(u, -limit, limit): g' * sigmoid(alpha g') * (u' + shift).
+// `silu` is the product's own form of silu(g) * u, so that the plain unit's results stay what they were.
+template <typename Silu>
+__device__ __forceinline__ float fw_gated_unit(float g, float u, float limit, float alpha, float shift, Silu silu) {
+    if (limit <= 0.0f) return silu(g) * u;
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+    const float z = alpha * g;
+    const float e = __expf(z >= 0.0f ? -z : z);
+    return g * (z >= 0.0f ? 1.0f / (1.0f + e) : e / (1.0f + e)) * (u + shift);
+}
+
 static inline int fw_ceil_div(long long a, long long b) { return (int)((a + b - 1) / b); }
 
 // Eight bfloat16 of a weight matrix that a decode step reads once: with `streamed` the load says

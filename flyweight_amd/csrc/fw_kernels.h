@@ -75,7 +75,7 @@ int fw_gemm_medium(const void* a, const void* w, int w_tiled, const float* bias,
                    int M, int N, int K, void* workspace, size_t workspace_bytes, int* counters,
                    int counters_len, const float* next_norm_weight, int next_one_centered,
                    void* next_activations, float* next_squares, const float* squares, int squares_rows,
-                   float eps, void* stream);
+                   float eps, float glu_limit, float glu_alpha, float glu_shift, void* stream);
 
 // Fused product for decode steps of up to 16 rows. prologue 0: a is bfloat16 [M][K]; 1: a is
 // float32 rows, RMS-normed with norm_weight/eps (rows gathered through row_index if given) inside
@@ -87,6 +87,9 @@ int fw_gemm_medium(const void* a, const void* w, int w_tiled, const float* bias,
 // [M][N] = x_new * w_next and next_squares [fw_gemm_decode_accumulate_tiles(N)][16], per-tile sums
 // of x_new^2 of every row. A later call takes them with prologue 2 (a = those activations,
 // squares/squares_tiles = those sums, eps) and applies the row's scale in its epilogue.
+// glu_limit / glu_alpha / glu_shift (here and in fw_gemm_medium, epilogue 2 only): with a limit <= 0 the
+// gated unit is SwiGLU, silu(gate) * up; with a positive one its halves are clamped, g = min(gate,
+// limit), u = clamp(up, -limit, limit), and out = g * sigmoid(alpha * g) * (u + shift).
 // w_tiled (here and in fw_gemm_medium): w is not row-major [rows][K] but lies in operand tiles,
 // [rows / 16][K / 32][4][16][8]: tile (i, j) holds rows 16 i .. 16 i + 15, columns 32 j .. 32 j + 31 as
 // 1 KB in the order in which a wave loads a matrix-core operand (lane = 16 * (column / 8) + row), so
@@ -97,7 +100,7 @@ int fw_gemm_decode(int prologue, const void* a, const float* norm_weight, const 
                    int M, int N, int K, const float* taps, const float* conv_bias, float* state,
                    const int32_t* seg_slot, int kernel_size, const float* next_norm_weight,
                    int next_one_centered, void* next_activations, float* next_squares, const float* squares,
-                   int squares_tiles, void* stream);
+                   int squares_tiles, float glu_limit, float glu_alpha, float glu_shift, void* stream);
 int fw_gemm_decode_fits(int M, int N, int K, int epilogue);
 int fw_gemm_decode_accumulate_tiles(int N);
 
@@ -137,7 +140,8 @@ int fw_attention_generic(const void* q, void* out, int dtype, const void* k_page
                          int num_kv_heads, int head_dim, int v_dim, float scale, int window, int page_size,
                          int num_pages, void* stream);
 
-// The same attention on the matrix cores, bfloat16 only, head_dim a multiple of 16 up to 256.
+// The same attention on the matrix cores, bfloat16 only, head_dim and v_dim (the size of a value and of a
+// head's output: out [rows][nh * v_dim]) multiples of 16 up to 256.
 // Prompt portions: rows are cut into tiles of up to 64 that never span two segments (tile_seg,
 // tile_row0), in any order: workgroups start in the order of the tiles, so the caller lists those
 // that see the most keys first. heads_together: how many query heads of a kv group one workgroup takes, reading
@@ -146,11 +150,11 @@ int fw_attention_generic(const void* q, void* out, int dtype, const void* k_page
 int fw_attention_prefill(const void* q, void* out, const void* k_pages, const void* v_pages,
                          const int32_t* block_table, int table_stride, const int32_t* tile_seg,
                          const int32_t* tile_row0, int tiles, const int32_t* seg_row0, const int32_t* row_pos,
-                         int rows, int num_heads, int num_kv_heads, int head_dim, float scale, int window,
+                         int rows, int num_heads, int num_kv_heads, int head_dim, int v_dim, float scale, int window,
                          int page_size, int num_pages, int heads_together, void* stream);
 // Decode (one row per request): the keys are split between workgroups in runs of 4 pages and
 // merged in order by the workgroup that finishes last. partial: float32 workspace
-// [rows][heads][max_splits][head_dim + 4]; max_context: an upper bound on position + 1 of every
+// [rows][heads][max_splits][v_dim + 4]; max_context: an upper bound on position + 1 of every
 // row, known to the caller; tickets: rows * kv_heads * ceil(heads / kv_heads / 16) int32 counters,
 // zero before the first call and left zero. decode_work: null, or one int32 on the device, the runs
 // of 4 pages that all the rows of the step see together; with it a workgroup takes as many runs as
@@ -158,10 +162,10 @@ int fw_attention_prefill(const void* q, void* out, const void* k_pages, const vo
 int fw_attention_decode(const void* q, void* out, float* partial, int max_splits, int max_context,
                         const int32_t* decode_work, int* tickets, int tickets_len, const void* k_pages, const void* v_pages, const int32_t* block_table, int table_stride,
                         const int32_t* row_seg, const int32_t* row_pos, int rows, int num_heads, int num_kv_heads,
-                        int head_dim, float scale, int window, int page_size, int num_pages, void* stream);
+                        int head_dim, int v_dim, float scale, int window, int page_size, int num_pages, void* stream);
 
 // The same with the work of fw_qk_norm_rope_kv_write in front of it, in one kernel: qkv float32
-// [rows][(heads + 2 kv_heads) * head_dim] are the step's raw projections; every workgroup norms and
+// [rows][(heads + kv_heads) * head_dim + kv_heads * v_dim] are the step's raw projections; every workgroup norms and
 // rotates the query heads it works on, and the one whose pages hold the row's own position stores
 // the new key (normed, rotated) and value (write_kv 0: they are in the cache already).
 int fw_attention_decode_fused(const float* qkv, const float* q_norm_weight, const float* k_norm_weight, float eps,
@@ -169,8 +173,8 @@ int fw_attention_decode_fused(const float* qkv, const float* q_norm_weight, cons
                               float* partial, int max_splits, int max_context, const int32_t* decode_work, int* tickets,
                               int tickets_len, void* k_pages,
                               void* v_pages, const int32_t* block_table, int table_stride, const int32_t* row_seg,
-                              const int32_t* row_pos, int rows, int num_heads, int num_kv_heads, int head_dim, float scale,
-                              int window, int page_size, int num_pages, void* stream);
+                              const int32_t* row_pos, int rows, int num_heads, int num_kv_heads, int head_dim, int v_dim,
+                              float scale, int window, int page_size, int num_pages, void* stream);
 
 // ids[r] = argmax(logits[r]) with ties to the lowest id, also written to also[r] if that is not null;
 // advance[r] += 1 if that is not null; workspace: rows * 64 64-bit words

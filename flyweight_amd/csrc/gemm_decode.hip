@@ -64,6 +64,8 @@ struct DecodeGemmArgs {
     // pre-normed prologue
     const float* squares;           // [squares_tiles][16], left by the kernel above
     int squares_tiles;
+    // the gated unit of epilogue 2: limit <= 0: silu(gate) * up; else clamped halves (fw_gated_unit)
+    float glu_limit, glu_alpha, glu_shift;
 };
 
 __device__ __forceinline__ float dg_silu(float g) {
@@ -295,7 +297,8 @@ __global__ __launch_bounds__(WAVES * 64) void decode_gemm_kernel(const DecodeGem
                     if (p.bias) total[rt][r] += p.bias[n + rt * p.tile_stride];
                 }
                 if (EPI == DG_SWIGLU) {
-                    store_from_float(out, (size_t)m * N + n, dg_silu(total[0][r]) * total[RT > 1 ? 1 : 0][r]);
+                    store_from_float(out, (size_t)m * N + n, fw_gated_unit(total[0][r], total[RT > 1 ? 1 : 0][r], p.glu_limit, p.glu_alpha,
+                                                                           p.glu_shift, [](float g) { return dg_silu(g); }));
                 } else {        // DG_CONV: tiles are B, C, x of channel n; the row is a segment of one token
                     const int history = p.kernel_size - 1;
                     float* channel_state = p.state + ((size_t)conv_slot * N + n) * history;
@@ -358,7 +361,8 @@ extern "C" int fw_gemm_decode(int prologue, const void* a, const float* norm_wei
                               int out_dtype, int epilogue, int M, int N, int K, const float* taps,
                               const float* conv_bias, float* state, const int32_t* seg_slot, int kernel_size,
                               const float* next_norm_weight, int next_one_centered, void* next_activations,
-                              float* next_squares, const float* squares, int squares_tiles, void* stream) {
+                              float* next_squares, const float* squares, int squares_tiles, float glu_limit, float glu_alpha,
+                              float glu_shift, void* stream) {
     FW_REQUIRE(M >= 1 && M <= 16, "gemm_decode: takes 1..16 rows, got %d", M);
     FW_REQUIRE(N > 0 && K > 0 && K % 8 == 0, "gemm_decode: K (%d) must be a positive multiple of 8, N (%d) positive", K, N);
     FW_REQUIRE(prologue >= 0 && prologue <= 2, "gemm_decode: unknown prologue %d", prologue);
@@ -385,6 +389,7 @@ extern "C" int fw_gemm_decode(int prologue, const void* a, const float* norm_wei
     args.next_norm_weight = next_norm_weight; args.next_one_centered = next_one_centered;
     args.next_activations = (uint16_t*)next_activations; args.next_squares = next_squares;
     args.squares = squares; args.squares_tiles = squares_tiles;
+    args.glu_limit = glu_limit; args.glu_alpha = glu_alpha; args.glu_shift = glu_shift;
     hipStream_t s = (hipStream_t)stream;
     // Few features: tiles of 8, so that there are more workgroups (2,048 features: 256 instead of 128). From 192
     // tiles of 16 on the wider tile wins, whose waves read whole 1 KB pieces of W (3,072 features at 8 rows: 4.9

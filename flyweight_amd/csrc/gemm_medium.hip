@@ -56,6 +56,8 @@ struct MediumArgs {
     int squares_rows;
     float eps;
     int rotate;                     // workgroups start their walk over K at different chunks
+    // the gated unit of mode 2: limit <= 0: silu(gate) * up; else clamped halves (fw_gated_unit)
+    float glu_limit, glu_alpha, glu_shift;
 };
 
 // rows of the sums of squares are 16 wide for up to 16 rows of a (the fused decode product's
@@ -327,7 +329,8 @@ __global__ __launch_bounds__(GM_THREADS) void gemm_medium_kernel(const MediumArg
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const int n = n_first + r;
-            if (MODE == GM_SWIGLU) v[r] = gm_silu(acc[0][mt][r] * inv) * (acc[1][mt][r] * inv);
+            if (MODE == GM_SWIGLU) v[r] = fw_gated_unit(acc[0][mt][r] * inv, acc[1][mt][r] * inv, p.glu_limit, p.glu_alpha, p.glu_shift,
+                                                        [](float g) { return gm_silu(g); });
             else v[r] = acc[0][mt][r] * inv + ((p.bias && n < N) ? p.bias[n] : 0.0f);
         }
         if (mine) {
@@ -471,7 +474,7 @@ extern "C" int fw_gemm_medium(const void* a, const void* w, int w_tiled, const f
                               int M, int N, int K, void* workspace, size_t workspace_bytes, int* counters,
                               int counters_len, const float* next_norm_weight, int next_one_centered,
                               void* next_activations, float* next_squares, const float* squares, int squares_rows,
-                              float eps, void* stream) {
+                              float eps, float glu_limit, float glu_alpha, float glu_shift, void* stream) {
     FW_REQUIRE(M >= 1 && M <= 64, "gemm_medium: takes 1..64 rows, got %d", M);
     FW_REQUIRE(N > 0 && K > 0 && K % 8 == 0, "gemm_medium: K (%d) must be a positive multiple of 8, N (%d) positive", K, N);
     FW_REQUIRE(mode >= 0 && mode <= 2, "gemm_medium: unknown mode %d", mode);
@@ -497,6 +500,7 @@ extern "C" int fw_gemm_medium(const void* a, const void* w, int w_tiled, const f
     args.next_norm_weight = next_norm_weight; args.next_one_centered = next_one_centered;
     args.next_activations = (uint16_t*)next_activations; args.next_squares = next_squares;
     args.squares = squares; args.squares_rows = squares_rows; args.eps = eps;
+    args.glu_limit = glu_limit; args.glu_alpha = glu_alpha; args.glu_shift = glu_shift;
     args.rotate = plan.splits == 1 && (long long)N * K * (mode == GM_SWIGLU ? 2 : 1) > (1ll << 24);
     const dim3 grid(plan.tiles, plan.splits);
     hipStream_t s = (hipStream_t)stream;

@@ -19,7 +19,7 @@ from . import build as _build
 F32, BF16 = 0, 1
 PAGE_SIZE = 64          # tokens per cache page: the width of a wavefront
 MAX_HEAD_DIM = 256
-ABI_VERSION = 10
+ABI_VERSION = 12
 
 _lib = None
 
@@ -615,7 +615,8 @@ def _tiled_for(w: torch.Tensor, w_tiled: Optional[torch.Tensor]) -> Optional[tor
 
 def gemm_medium_into(a: torch.Tensor, w: torch.Tensor, bias, target: torch.Tensor, out_code: int, mode: int, N: int,
                      next_norm_weight: Optional[torch.Tensor] = None, next_one_centered: bool = False,
-                     squares: Optional[torch.Tensor] = None, eps: float = 0.0, w_tiled: Optional[torch.Tensor] = None):
+                     squares: Optional[torch.Tensor] = None, eps: float = 0.0, w_tiled: Optional[torch.Tensor] = None,
+                     glu: Optional[tuple] = None):
     """The product for 1..64 rows with K split over workgroups (fw_gemm_medium). With
     ``squares`` ``a`` holds prepared activations (x * w of an RMS norm) and the rows' 1/rms is
     formed from those sums. With ``next_norm_weight`` (accumulating product) returns what the
@@ -640,7 +641,7 @@ def gemm_medium_into(a: torch.Tensor, w: torch.Tensor, bias, target: torch.Tenso
                                     ctypes.c_size_t(need_bytes.value), _p(counters),
                                     0 if counters is None else counters.numel(), _p(next_norm_weight),
                                     int(next_one_centered), _p(next_activations), _p(next_squares), _p(squares),
-                                    0 if squares is None else squares.shape[0], ctypes.c_float(eps), _stream()))
+                                    0 if squares is None else squares.shape[0], ctypes.c_float(eps), *_glu(glu), _stream()))
     if next_norm_weight is not None:
         return next_activations, next_squares
     return None
@@ -650,10 +651,11 @@ def gemm_medium(a: torch.Tensor, w: torch.Tensor, epilogue: int, *, bias: Option
                 out_dtype: Optional[torch.dtype] = None, accumulate_into: Optional[torch.Tensor] = None,
                 squares: Optional[torch.Tensor] = None, eps: float = 0.0,
                 next_norm_weight: Optional[torch.Tensor] = None, next_one_centered: bool = False,
-                w_tiled: Optional[torch.Tensor] = None):
+                w_tiled: Optional[torch.Tensor] = None, glu: Optional[tuple] = None):
     """The medium product with the fused decode product's conventions (EPILOGUE_STORE /
     ACCUMULATE / SWIGLU): returns the output, or for an accumulation with ``next_norm_weight``
-    what the norm after it needs."""
+    what the norm after it needs. ``glu`` (with EPILOGUE_SWIGLU): (limit, alpha, shift) of a gated
+    unit with clamped halves instead of SwiGLU."""
     _dev(a, w, bias, accumulate_into, squares, next_norm_weight)
     _want(a, torch.bfloat16, "a")
     _want(w, torch.bfloat16, "w")
@@ -675,7 +677,7 @@ def gemm_medium(a: torch.Tensor, w: torch.Tensor, epilogue: int, *, bias: Option
         return accumulate_into if left is None else left
     out_dtype = torch.bfloat16 if epilogue == EPILOGUE_SWIGLU else (out_dtype or torch.bfloat16)
     out = torch.empty((M, N), dtype=out_dtype, device=a.device)
-    gemm_medium_into(a, w, bias, out, _code(out_dtype), epilogue, N, squares=squares, eps=eps, w_tiled=w_tiled)
+    gemm_medium_into(a, w, bias, out, _code(out_dtype), epilogue, N, squares=squares, eps=eps, w_tiled=w_tiled, glu=glu)
     return out
 
 
@@ -754,6 +756,16 @@ def gemm_swiglu(a: torch.Tensor, w_gate_up: torch.Tensor, w_tiled: Optional[torc
 
 # ---- fused products for decode steps of up to 16 rows --------------------------------------------
 EPILOGUE_STORE, EPILOGUE_ACCUMULATE, EPILOGUE_SWIGLU, EPILOGUE_CONV = 0, 1, 2, 3
+
+
+def _glu(glu: Optional[tuple]):
+    """The three numbers a gated epilogue takes: (0, 1, 0) is SwiGLU; else (limit > 0, alpha, shift)."""
+    if glu is None:
+        return ctypes.c_float(0.0), ctypes.c_float(1.0), ctypes.c_float(0.0)
+    limit, alpha, shift = glu
+    if not limit > 0:
+        raise KernelError("a gated unit with clamped halves needs a positive limit")
+    return ctypes.c_float(limit), ctypes.c_float(alpha), ctypes.c_float(shift)
 DECODE_MAX_ROWS = 16
 LONG_K = 4096
 LONG_K_TILED_ROWS = 8
@@ -770,8 +782,9 @@ def gemm_decode(a: torch.Tensor, w: torch.Tensor, epilogue: int, *, bias: Option
                 conv_bias: Optional[torch.Tensor] = None, state: Optional[torch.Tensor] = None,
                 seg_slot: Optional[torch.Tensor] = None, squares: Optional[torch.Tensor] = None,
                 next_norm_weight: Optional[torch.Tensor] = None, next_one_centered: bool = False,
-                w_tiled: Optional[torch.Tensor] = None):
+                w_tiled: Optional[torch.Tensor] = None, glu: Optional[tuple] = None):
     """One kernel for (optional RMS norm of float32 rows) -> product with bfloat16 ``w`` -> epilogue.
+    ``glu`` (with EPILOGUE_SWIGLU): (limit, alpha, shift) of a gated unit with clamped halves.
     With ``norm_weight`` ``a`` holds float32 rows (gathered through ``row_index`` if given), else
     bfloat16 activations. With ``next_norm_weight`` the accumulating epilogue also leaves what
     the norm after it needs, and the call returns (activations x * w_next, sums of squares);
@@ -838,7 +851,7 @@ def gemm_decode(a: torch.Tensor, w: torch.Tensor, epilogue: int, *, bias: Option
         _p(w if w_tiled is None else w_tiled), int(w_tiled is not None), _p(bias),
         _p(target), _code(out_dtype), int(epilogue), rows, N, K, _p(taps), _p(conv_bias), _p(state), _p(seg_slot),
         int(kernel_size), _p(next_norm_weight), int(next_one_centered), _p(next_activations), _p(next_squares),
-        _p(squares), 0 if squares is None else squares.shape[0], _stream()))
+        _p(squares), 0 if squares is None else squares.shape[0], *_glu(glu), _stream()))
     if next_norm_weight is not None:
         return next_activations, next_squares
     return target
@@ -872,27 +885,28 @@ def decode_splits(max_context: int, window: int = 0) -> int:
 def attention_prefill(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, k_pages: torch.Tensor,
                       v_pages: torch.Tensor, block_table: torch.Tensor, tile_seg: torch.Tensor, tile_row0: torch.Tensor,
                       seg_row0: torch.Tensor, row_pos: torch.Tensor, scale: float, window: int = 0,
-                      heads_together: int = 0, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                      heads_together: int = 0, out: Optional[torch.Tensor] = None, v_dim: Optional[int] = None) -> torch.Tensor:
     """``heads_together``: query heads of a kv group per workgroup (1, or 4 up to head_dim 64), 0: the
     kernel's choice. Only the rows of the given tiles are written (into ``out`` if given)."""
     _dev(q, k_pages, v_pages, block_table, tile_seg, tile_row0, seg_row0, row_pos)
     _want(q, torch.bfloat16, "q")
     rows = q.shape[0]
+    v_dim = head_dim if v_dim is None else int(v_dim)
     if q.shape != (rows, num_heads * head_dim):
         raise KernelError(f"attention: q is {tuple(q.shape)}, expected {(rows, num_heads * head_dim)}")
-    pages = _check_pages(k_pages, v_pages, num_kv_heads, head_dim, torch.bfloat16)
+    pages = _check_pages(k_pages, v_pages, num_kv_heads, head_dim, torch.bfloat16, v_dim)
     for name, t in (("block_table", block_table), ("tile_seg", tile_seg), ("tile_row0", tile_row0),
                     ("seg_row0", seg_row0), ("row_pos", row_pos)):
         _want(t, torch.int32, name)
     if block_table.dim() != 2 or row_pos.numel() < rows or tile_seg.numel() != tile_row0.numel():
         raise KernelError("attention: batch index arrays are inconsistent")
     if out is None:
-        out = torch.empty_like(q)
-    elif out.shape != q.shape or out.dtype != q.dtype or not out.is_contiguous():
-        raise KernelError("attention: out must be like q")
+        out = torch.empty((rows, num_heads * v_dim), dtype=q.dtype, device=q.device)
+    elif out.shape != (rows, num_heads * v_dim) or out.dtype != q.dtype or not out.is_contiguous():
+        raise KernelError("attention: out must be bfloat16 [rows, heads * v_dim]")
     _check(library().fw_attention_prefill(
         _p(q), _p(out), _p(k_pages), _p(v_pages), _p(block_table), block_table.shape[1], _p(tile_seg), _p(tile_row0),
-        tile_seg.numel(), _p(seg_row0), _p(row_pos), rows, num_heads, num_kv_heads, head_dim, ctypes.c_float(scale),
+        tile_seg.numel(), _p(seg_row0), _p(row_pos), rows, num_heads, num_kv_heads, head_dim, v_dim, ctypes.c_float(scale),
         int(window), PAGE_SIZE, pages, int(heads_together), _stream()))
     return out
 
@@ -909,7 +923,7 @@ def _work(decode_work: Optional[torch.Tensor]):
 def attention_decode(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, k_pages: torch.Tensor,
                      v_pages: torch.Tensor, block_table: torch.Tensor, row_seg: torch.Tensor, row_pos: torch.Tensor,
                      scale: float, max_context: int, window: int = 0, out: Optional[torch.Tensor] = None,
-                     decode_work: Optional[torch.Tensor] = None) -> torch.Tensor:
+                     decode_work: Optional[torch.Tensor] = None, v_dim: Optional[int] = None) -> torch.Tensor:
     """One row per request; ``max_context`` bounds position + 1 of every row (the host knows it).
     ``decode_work``: one int32 on the device, the runs of 4 pages that the rows see together (the
     sum of ceil((position + 1) / 256)): the kernel shares the work out by it (fewer, longer
@@ -917,25 +931,26 @@ def attention_decode(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_di
     _dev(q, k_pages, v_pages, block_table, row_seg, row_pos)
     _want(q, torch.bfloat16, "q")
     rows = q.shape[0]
+    v_dim = head_dim if v_dim is None else int(v_dim)
     if q.shape != (rows, num_heads * head_dim):
         raise KernelError(f"attention: q is {tuple(q.shape)}, expected {(rows, num_heads * head_dim)}")
-    pages = _check_pages(k_pages, v_pages, num_kv_heads, head_dim, torch.bfloat16)
+    pages = _check_pages(k_pages, v_pages, num_kv_heads, head_dim, torch.bfloat16, v_dim)
     for name, t in (("block_table", block_table), ("row_seg", row_seg), ("row_pos", row_pos)):
         _want(t, torch.int32, name)
     if block_table.dim() != 2 or row_seg.numel() < rows or row_pos.numel() < rows:
         raise KernelError("attention: batch index arrays are too short")
     splits = decode_splits(max_context, window)
-    partial = torch.empty((rows, num_heads, splits, head_dim + 4), dtype=torch.float32, device=q.device)
+    partial = torch.empty((rows, num_heads, splits, v_dim + 4), dtype=torch.float32, device=q.device)
     if out is None:
-        out = torch.empty_like(q)
-    elif out.shape != q.shape or out.dtype != q.dtype or not out.is_contiguous():
-        raise KernelError("attention: out must be like q")
+        out = torch.empty((rows, num_heads * v_dim), dtype=q.dtype, device=q.device)
+    elif out.shape != (rows, num_heads * v_dim) or out.dtype != q.dtype or not out.is_contiguous():
+        raise KernelError("attention: out must be bfloat16 [rows, heads * v_dim]")
     group = num_heads // num_kv_heads
     tickets = _medium_counters(q.device, rows * num_kv_heads * ((group + 15) // 16))
     _check(library().fw_attention_decode(
         _p(q), _p(out), _p(partial), splits, int(max_context), _work(decode_work), _p(tickets), tickets.numel(), _p(k_pages), _p(v_pages),
         _p(block_table),
-        block_table.shape[1], _p(row_seg), _p(row_pos), rows, num_heads, num_kv_heads, head_dim, ctypes.c_float(scale),
+        block_table.shape[1], _p(row_seg), _p(row_pos), rows, num_heads, num_kv_heads, head_dim, v_dim, ctypes.c_float(scale),
         int(window), PAGE_SIZE, pages, _stream()))
     return out
 
@@ -945,7 +960,7 @@ def attention_decode_fused(qkv: torch.Tensor, num_heads: int, num_kv_heads: int,
                            cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], rotary_dim: int, k_pages: torch.Tensor,
                            v_pages: torch.Tensor, block_table: torch.Tensor, row_seg: torch.Tensor, row_pos: torch.Tensor,
                            scale: float, max_context: int, window: int = 0, write_kv: bool = True,
-                           decode_work: Optional[torch.Tensor] = None) -> torch.Tensor:
+                           decode_work: Optional[torch.Tensor] = None, v_dim: Optional[int] = None) -> torch.Tensor:
     """One row per request, from the step's raw projections ``qkv`` (float32 [rows, (heads + 2 kv
     heads) * head_dim]): per-head norm and rotation of queries and keys, the new keys and values
     into their pages, and the split-key attention, in one kernel. Returns bfloat16 [rows, heads *
@@ -953,9 +968,10 @@ def attention_decode_fused(qkv: torch.Tensor, num_heads: int, num_kv_heads: int,
     _dev(qkv, q_norm_weight, k_norm_weight, cos, sin, k_pages, v_pages, block_table, row_seg, row_pos)
     _want(qkv, torch.float32, "qkv")
     rows, width = qkv.shape
-    if width != (num_heads + 2 * num_kv_heads) * head_dim:
-        raise KernelError(f"attention_decode_fused: qkv width {width} != ({num_heads} + 2 x {num_kv_heads}) x {head_dim}")
-    pages = _check_pages(k_pages, v_pages, num_kv_heads, head_dim, torch.bfloat16)
+    v_dim = head_dim if v_dim is None else int(v_dim)
+    if width != (num_heads + num_kv_heads) * head_dim + num_kv_heads * v_dim:
+        raise KernelError(f"attention_decode_fused: qkv width {width} != ({num_heads} + {num_kv_heads}) x {head_dim} + {num_kv_heads} x {v_dim}")
+    pages = _check_pages(k_pages, v_pages, num_kv_heads, head_dim, torch.bfloat16, v_dim)
     for w in (q_norm_weight, k_norm_weight):
         if w is not None:
             _want(w, torch.float32, "norm weight")
@@ -971,14 +987,14 @@ def attention_decode_fused(qkv: torch.Tensor, num_heads: int, num_kv_heads: int,
     if block_table.dim() != 2 or row_seg.numel() < rows or row_pos.numel() < rows:
         raise KernelError("attention: batch index arrays are too short")
     splits = decode_splits(max_context, window)
-    partial = torch.empty((rows, num_heads, splits, head_dim + 4), dtype=torch.float32, device=qkv.device)
-    out = torch.empty((rows, num_heads * head_dim), dtype=torch.bfloat16, device=qkv.device)
+    partial = torch.empty((rows, num_heads, splits, v_dim + 4), dtype=torch.float32, device=qkv.device)
+    out = torch.empty((rows, num_heads * v_dim), dtype=torch.bfloat16, device=qkv.device)
     group = num_heads // num_kv_heads
     tickets = _medium_counters(qkv.device, rows * num_kv_heads * ((group + 15) // 16))
     _check(library().fw_attention_decode_fused(
         _p(qkv), _p(q_norm_weight), _p(k_norm_weight), ctypes.c_float(eps), _p(cos), _p(sin), int(rotary_dim), int(write_kv), _p(out),
         _p(partial), splits, int(max_context), _work(decode_work), _p(tickets), tickets.numel(), _p(k_pages), _p(v_pages), _p(block_table),
-        block_table.shape[1], _p(row_seg), _p(row_pos), rows, num_heads, num_kv_heads, head_dim, ctypes.c_float(scale), int(window),
+        block_table.shape[1], _p(row_seg), _p(row_pos), rows, num_heads, num_kv_heads, head_dim, v_dim, ctypes.c_float(scale), int(window),
         PAGE_SIZE, pages, _stream()))
     return out
 
@@ -998,12 +1014,13 @@ def attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
     would hold a 64-row tile of the prompt kernel and walk its whole context alone), the tiled
     kernel for the rest (``tile_seg``, ``tile_row0``: the tiles of ``query_tiles`` in the order
     workgroups take them, those of the leading single rows in front; ``decode_work``: see
-    ``attention_decode``); float32, value heads of another size than the keys' (``v_dim``) and
-    everything else on the generic kernel."""
-    fast = q.dtype == torch.bfloat16 and attention_is_tiled(head_dim) and v_dim in (None, head_dim)
+    ``attention_decode``); float32 and everything else on the generic kernel. ``v_dim``: the size of a
+    value head (and of a head's output) where it is not ``head_dim``."""
+    v_dim = head_dim if v_dim is None else int(v_dim)
+    fast = q.dtype == torch.bfloat16 and attention_is_tiled(head_dim) and attention_is_tiled(v_dim)
     if fast and ctx.all_decode:
         return attention_decode(q, num_heads, num_kv_heads, head_dim, k_pages, v_pages, block_table, ctx.row_seg,
-                                ctx.row_pos, scale, ctx.max_context, window, decode_work=decode_work)
+                                ctx.row_pos, scale, ctx.max_context, window, decode_work=decode_work, v_dim=v_dim)
     if fast:
         if tile_seg is None or tile_row0 is None:
             raise KernelError("attention: the tiled kernel needs the step's query tiles")
@@ -1013,16 +1030,16 @@ def attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
         # gives more and shorter workgroups, which evens out the causal triangle
         rows = q.shape[0] - single
         keys = min(window, ctx.max_context) if window else ctx.max_context      # the most keys a row can see
-        together = 4 if head_dim <= 64 and num_heads // num_kv_heads >= 4 and keys >= 4 * rows else 0
+        together = 4 if max(head_dim, v_dim) <= 64 and num_heads // num_kv_heads >= 4 and keys >= 4 * rows else 0
         if single == 0:
             return attention_prefill(q, num_heads, num_kv_heads, head_dim, k_pages, v_pages, block_table, tile_seg,
-                                     tile_row0, ctx.seg_row0, ctx.row_pos, scale, window, heads_together=together)
-        out = torch.empty_like(q)
+                                     tile_row0, ctx.seg_row0, ctx.row_pos, scale, window, heads_together=together, v_dim=v_dim)
+        out = torch.empty((q.shape[0], num_heads * v_dim), dtype=q.dtype, device=q.device)
         attention_decode(q[:single], num_heads, num_kv_heads, head_dim, k_pages, v_pages, block_table, ctx.row_seg,
-                         ctx.row_pos, scale, ctx.max_context, window, out=out[:single], decode_work=decode_work)
+                         ctx.row_pos, scale, ctx.max_context, window, out=out[:single], decode_work=decode_work, v_dim=v_dim)
         return attention_prefill(q, num_heads, num_kv_heads, head_dim, k_pages, v_pages, block_table,
                                  tile_seg[single:], tile_row0[single:], ctx.seg_row0, ctx.row_pos, scale, window,
-                                 heads_together=together, out=out)
+                                 heads_together=together, out=out, v_dim=v_dim)
     return attention_generic(q, num_heads, num_kv_heads, head_dim, k_pages, v_pages, block_table, ctx.row_seg,
                              ctx.row_pos, scale, window, v_dim=v_dim)
 

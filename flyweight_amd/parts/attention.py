@@ -110,7 +110,7 @@ class GQAttention(Mixer):
 
     def step_arrays_key(self):
         fast = getattr(self, "dtype", None) == torch.bfloat16 and ops.attention_is_tiled(self.head_dim) \
-            and self.v_head_dim == self.head_dim
+            and ops.attention_is_tiled(self.v_head_dim)
         return ("query_tiles", ops.QUERY_TILE, self.RUN_OF_KEYS) if fast else None
 
     def _decode_work(self, batch) -> int:
@@ -149,7 +149,7 @@ class GQAttention(Mixer):
                 qkv, self.num_heads, self.num_kv_heads, self.head_dim, self.q_norm_weight, self.k_norm_weight, self.qk_norm_eps,
                 cos, sin, self.position.rotary_dim, cache.k_pages, cache.v_pages, cache.block_table, ctx.row_seg, ctx.row_pos,
                 self.scale, ctx.max_context, int(self.window or 0), write_kv=cache.writes,
-                decode_work=own.get("decode_work"))
+                decode_work=own.get("decode_work"), v_dim=self.v_head_dim)
         q = ops.qk_norm_rope_kv_write(
             qkv, self.num_heads, self.num_kv_heads, self.head_dim, self.q_norm_weight, self.k_norm_weight,
             self.qk_norm_eps, cos, sin, self.position.rotary_dim, cache.k_pages, cache.v_pages, cache.block_table,

@@ -52,7 +52,7 @@ class ClampedGLU(FeedForward):
         self.down = Linear(tensors[self._name("down")])
 
     def activation(self, h) -> torch.Tensor:
-        return ops.clamped_glu(self.gate_up.forward(h, out_dtype=torch.float32), self.limit, self.alpha, self.shift, self.dtype)
+        return self.gate_up.clamped_glu(h, self.limit, self.alpha, self.shift)
 
     def output_terms(self, h, ctx) -> List[Tuple[torch.Tensor, float]]:
         return [(self.down.forward(self.activation(h), out_dtype=torch.float32), 1.0)]

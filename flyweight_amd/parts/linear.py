@@ -145,6 +145,18 @@ class Linear:
                                    w_tiled=self.tiled, **self._norm_arguments(a))
         return ops.gemm_swiglu(self._tensor_of(a), self.weight, w_tiled=self.tiled)
 
+    def clamped_glu(self, a: Input, limit: float, alpha: float, shift: float) -> torch.Tensor:
+        """The weight holds gate rows then up rows: g * sigmoid(alpha g) * (u + shift) with g = min(gate,
+        limit), u = clamp(up, -limit, limit). In the products of few rows the unit is the product's
+        epilogue, as SwiGLU is; a prompt's product leaves float32 sums and a kernel of its own forms it."""
+        if self.bias is None and self._medium(a):
+            return ops.gemm_medium(self._rows_of(a), self.weight, ops.EPILOGUE_SWIGLU, w_tiled=self.tiled, glu=(limit, alpha, shift),
+                                   **self._prepared_arguments(a))
+        if self.bias is None and self._fused(a, self.out_features // 2, ops.EPILOGUE_SWIGLU):
+            return ops.gemm_decode(self._rows_of(a), self.weight, ops.EPILOGUE_SWIGLU, out_dtype=torch.bfloat16,
+                                   w_tiled=self.tiled, glu=(limit, alpha, shift), **self._norm_arguments(a))
+        return ops.clamped_glu(self.forward(a, out_dtype=torch.float32), limit, alpha, shift, a.dtype)
+
     def short_conv_decode(self, a: Input, taps: torch.Tensor, conv_bias: Optional[torch.Tensor], state: torch.Tensor,
                           seg_slot: torch.Tensor, out_dtype: torch.dtype) -> Optional[torch.Tensor]:
         """For single-token segments: the weight holds B, C and x rows; returns C * conv(B * x)

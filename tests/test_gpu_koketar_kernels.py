@@ -192,3 +192,68 @@ def test_attention_with_values_of_their_own_size(dtype):
             weight = np.exp(score - score.max())
             want = (weight / weight.sum()) @ v[lo:i + 1, 0]
             np.testing.assert_allclose(got[i, head], want, atol=1e-4 if dtype == "float32" else 3e-2, err_msg=f"row {i} back {back[i]}")
+
+
+@pytest.mark.parametrize("head_dim,v_dim", [(16, 48), (64, 128), (128, 64), (48, 16), (32, 32)])
+@pytest.mark.parametrize("window", [0, 70])
+def test_matrix_core_attention_with_values_of_their_own_size(head_dim, v_dim, window):
+    """The tiled prompt kernel, the split-key decode kernel and the decode kernel that norms, rotates
+    and stores on its way, against the generic kernel on the same pages (bfloat16): keys and values of
+    different sizes, queries made to match single keys near the window's edge and at page borders."""
+    from flyweight_amd.kernels import ops
+    rng = np.random.default_rng(head_dim * 7 + v_dim)
+    heads, kv_heads, scale, rows = 4, 2, 0.7, 200
+    k = plain.unit(rng.normal(size=(rows + 1, kv_heads, head_dim))) * 3.0
+    v = rng.normal(size=(rows + 1, kv_heads, v_dim))
+    back = rng.choice([0, 1, 63, 64, 65, 68, 69, 70, 71], size=rows + 1)
+    q = np.stack([np.stack([k[max(0, i - back[i]), h // 2] * 2.0 for h in range(heads)]) for i in range(rows + 1)])
+    qkv = np.concatenate([q.reshape(rows + 1, -1), k.reshape(rows + 1, -1), v.reshape(rows + 1, -1)], axis=1)
+    pages = 6
+    k_pages = torch.zeros((pages, kv_heads, 64, head_dim), dtype=torch.bfloat16, device="cuda")
+    v_pages = torch.zeros((pages, kv_heads, v_dim, 64), dtype=torch.bfloat16, device="cuda")
+    v_pages.fill_(9.0)          # what an earlier owner left behind the sequence's end must not count
+    table = ints([5, 0, 3, 1]).view(1, 4)
+    row_seg, row_pos = ints([0] * rows), ints(range(rows))
+    q_rows = ops.qk_norm_rope_kv_write(dev(qkv[:rows]), heads, kv_heads, head_dim, None, None, 1.0, None, None, 0, k_pages, v_pages,
+                                       table, row_seg, row_pos, v_dim=v_dim)
+    want = ops.attention_generic(q_rows, heads, kv_heads, head_dim, k_pages, v_pages, table, row_seg, row_pos, scale, window, v_dim=v_dim)
+    tile_seg, tile_row0 = ops.query_tiles([0, rows])
+    got = ops.attention_prefill(q_rows, heads, kv_heads, head_dim, k_pages, v_pages, table, ints(tile_seg), ints(tile_row0),
+                                ints([0, rows]), row_pos, scale, window, v_dim=v_dim)
+    assert got.shape == (rows, heads * v_dim)
+    np.testing.assert_allclose(got.float().cpu().numpy(), want.float().cpu().numpy(), atol=4e-2, rtol=2e-2)
+    # one row per request: the rows at positions 130 and 199 of the same sequence, as two requests on the same pages
+    two = ints([130, 199])
+    both_tables = table.repeat(2, 1).contiguous()
+    got = ops.attention_decode(q_rows[[130, 199]].contiguous(), heads, kv_heads, head_dim, k_pages, v_pages, both_tables, ints([0, 1]), two,
+                               scale, 256, window, v_dim=v_dim)
+    np.testing.assert_allclose(got.float().cpu().numpy(), want[[130, 199]].float().cpu().numpy(), atol=4e-2, rtol=2e-2)
+    # the next token from its raw projections: stored and attended in one kernel, against the two kernels on a copy
+    k_copy, v_copy = k_pages.clone(), v_pages.clone()
+    last = dev(qkv[rows:rows + 1])
+    q_last = ops.qk_norm_rope_kv_write(last, heads, kv_heads, head_dim, None, None, 1.0, None, None, 0, k_copy, v_copy, table,
+                                       ints([0]), ints([rows]), v_dim=v_dim)
+    want_last = ops.attention_generic(q_last, heads, kv_heads, head_dim, k_copy, v_copy, table, ints([0]), ints([rows]), scale, window, v_dim=v_dim)
+    got_last = ops.attention_decode_fused(last, heads, kv_heads, head_dim, None, None, 1.0, None, None, 0, k_pages, v_pages, table,
+                                          ints([0]), ints([rows]), scale, 256, window, v_dim=v_dim)
+    np.testing.assert_allclose(got_last.float().cpu().numpy(), want_last.float().cpu().numpy(), atol=4e-2, rtol=2e-2)
+    assert torch.equal(k_pages, k_copy) and torch.equal(v_pages, v_copy)
+
+
+@pytest.mark.parametrize("rows", [1, 8, 16, 40, 64, 200])
+def test_clamped_gated_unit_behind_its_product(rows):
+    """Few rows: the unit is the epilogue of the gate|up product (the decode product up to 16 rows, the
+    split-K product up to 64); more rows: float32 sums and the unit's own kernel. All against the plain formula."""
+    from flyweight_amd.parts.linear import Linear
+    rng = np.random.default_rng(rows)
+    hidden, inter, limit = 256, 384, 0.9
+    a = torch.from_numpy(rng.normal(size=(rows, hidden))).to(torch.bfloat16).cuda()
+    w = torch.from_numpy(rng.normal(size=(2 * inter, hidden)) / 8).to(torch.bfloat16).cuda()
+    got = Linear(w).clamped_glu(a, limit, 1.702, 1.0).float().cpu().numpy()
+    sums = a.double().cpu().numpy() @ w.double().cpu().numpy().T
+    gate, up = np.minimum(sums[:, :inter], limit), np.clip(sums[:, inter:], -limit, limit)
+    want = gate * plain.sigmoid(1.702 * gate) * (up + 1.0)
+    np.testing.assert_allclose(got, want, atol=1.5e-2, rtol=1e-2)
+    # the plain unit through the same products is what it was: silu(gate) * up
+    plain_unit = Linear(w).swiglu(a).float().cpu().numpy()
+    np.testing.assert_allclose(plain_unit, plain.silu(sums[:, :inter]) * sums[:, inter:], atol=3e-2, rtol=1.5e-2)
