@@ -55,7 +55,31 @@ CONFIG_Y = {
     ],
 }
 
-CONFIGS = {"X": CONFIG_X, "Y": CONFIG_Y}
+# Z: the corners. A window of one token (a row sees itself alone) and one wider than any prompt here; no
+# rotation at all and rotation of every channel; one tap (no convolution memory); heads of 4 and 8
+# channels; values narrower and wider than keys; one head on one key head and six on three; a
+# feed-forward width that is no multiple of eight (the products then take the plain kernel); a layer
+# without feed-forward; no soft cap; a factor of one on what joins the residual stream.
+CONFIG_Z = {
+    "architecture": "Koketar", "vocab": 97, "width": 40, "norm": {"eps": 1e-5}, "residual_mult": 1.0,
+    "layers": [
+        _layer(_left(1, 1, 8, 24, 1, 0, 10000.0, None, 1.0), _right(2, 2, 4, 4, 1, 3, 5), 0.7, 1.2, None, None),
+        _layer(_left(6, 3, 24, 8, 200, 24, 10000.0, 1.0, 0.25), _right(4, 1, 12, 20, 2, 8, 8), 1.0, 0.6, 50, 3.0),
+    ],
+}
+
+# W: wide enough that a prompt of some hundred tokens goes through the tiled prompt products and the
+# matrix-core attention (keys of 64, values of 128 channels and the other way round), with widths of
+# the joined operands that are no multiple of their tiles.
+CONFIG_W = {
+    "architecture": "Koketar", "vocab": 1000, "width": 512, "norm": {"eps": 1e-5}, "residual_mult": 0.4, "logit_softcap": 20.0,
+    "layers": [
+        _layer(_left(8, 2, 64, 128, 150, 32, 100000.0, 8.0, 0.125), _right(6, 3, 48, 80, 4, 24, 40), 0.8, 0.5, 1344, 1.0),
+        _layer(_left(4, 4, 128, 64, 90, 128, 100000.0, None, 0.09), _right(4, 4, 128, 128, 3, 16, 16), 1.0, 1.0, 1024, 2.0),
+    ],
+}
+
+CONFIGS = {"X": CONFIG_X, "Y": CONFIG_Y, "Z": CONFIG_Z, "W": CONFIG_W}
 
 # Largest difference from the plain float64 model, as a fraction of the largest logit compared, and
 # the same for the root mean square. float32 shows the logic right; the bfloat16 limits have to tell

@@ -62,7 +62,7 @@ def feed(stepper, request, tokens, cuts):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name", ["X", "Y"])
+@pytest.mark.parametrize("name", ["X", "Y", "Z"])
 def test_whole_prompt(models, name, dtype):
     loaded = models(name, dtype)
     tokens = random_tokens(loaded.config["vocab"], 200, seed=1)
@@ -76,7 +76,7 @@ def test_whole_prompt(models, name, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name", ["X", "Y"])
+@pytest.mark.parametrize("name", ["X", "Y", "Z"])
 def test_token_by_token_against_prefill(models, name, dtype):
     """Every token decoded alone, 170 steps: the windows (5, 33, 40, 64, 70 tokens) pass over decoded
     tokens and over page borders, the recurrences run on their carried state."""
@@ -99,6 +99,36 @@ def test_portions(models, name, dtype, cuts):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_a_wider_model_through_the_prompt_kernels(models, dtype):
+    """600 tokens of a model of width 512: whole (the tiled products, the matrix-core attention with keys
+    and values of different sizes), cut at odd places, and its last 40 tokens decoded one by one beside a
+    second request's portions (the products of few rows, the fused decode attention)."""
+    from flyweight_amd.engine import StepEntry
+    loaded = models("W", dtype)
+    tokens = random_tokens(loaded.config["vocab"], 600, seed=7)
+    other = random_tokens(loaded.config["vocab"], 300, seed=8)
+    expected = loaded.expected(tokens)
+    stepper = loaded.stepper(num_pages=26)
+    stepper.admit("whole")
+    assert_close(feed(stepper, "whole", tokens, [600]), expected, dtype, "W whole")
+    stepper.release("whole")
+    stepper.admit("cut")
+    assert_close(feed(stepper, "cut", tokens, [257, 17, 200, 63, 63]), expected, dtype, "W cut")
+    stepper.release("cut")
+    stepper.admit("a")
+    stepper.admit("b")
+    head = feed(stepper, "a", tokens[:560], [560])
+    rows, at = [], 0
+    for i in range(560, 600):
+        entries = [StepEntry("a", [tokens[i]], [0])]
+        if at < len(other):
+            entries.append(StepEntry("b", other[at:at + 9], []))
+            at += 9
+        rows.append(stepper.step(entries).cpu().numpy())
+    assert_close(np.concatenate([head] + rows), expected, dtype, "W decoded beside another request")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("variant", ["left", "right"])
 @pytest.mark.parametrize("name", ["X", "Y"])
 def test_each_branch_alone(models, name, variant, dtype):
@@ -112,7 +142,7 @@ def test_each_branch_alone(models, name, variant, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name", ["X", "Y"])
+@pytest.mark.parametrize("name", ["X", "Y", "Z"])
 def test_mixed_batches_on_few_pages_and_slots(models, name, dtype):
     """Eight requests of unequal length through four slots and a pool that holds four of them at
     most: portions of some beside single tokens of others, requests left out of steps, pages and slots
