@@ -185,8 +185,9 @@ __device__ __forceinline__ float delta_row_sum(float x) {
 }
 
 // Workgroup (segment, head, block of 16 value channels); thread = 16 * column + part: a column of S
-// is shared out over the 16 lanes of a row of the wave, RPT rows each (rows part * RPT .. + RPT - 1;
-// rows from dim on hold zeros), so that a head is spread over many compute units: the walk along the
+// is shared out over the 16 lanes of a row of the wave, RPT rows each (rows part, part + 16, ...: the
+// sixteen lanes then read sixteen neighbouring floats of q, k and g from LDS, one bank each; rows from
+// dim on hold zeros), so that a head is spread over many compute units: the walk along the
 // tokens is one dependent chain per column, and only its width can be bought. LDS per staged token:
 // q, k, g (16 * RPT each; past the record's padded dim they stay zero), beta and three unused, then the
 // block's 16 values. A thread copies the same pieces of every chunk (16-byte pieces: where each lies in
@@ -257,7 +258,7 @@ __global__ __launch_bounds__(256) void gated_delta_rule_kernel(
     float S[RPT];
 #pragma unroll
     for (int t = 0; t < RPT; ++t) {
-        const int i = part * RPT + t;
+        const int i = t * DELTA_LANES + part;
         S[t] = (live && i < dim) ? mine[i] : 0.0f;
     }
     __syncthreads();        // the zeros are in place
@@ -273,36 +274,37 @@ __global__ __launch_bounds__(256) void gated_delta_rule_kernel(
             const float* t0 = staged + token * TOKEN;
 #pragma unroll
             for (int t = 0; t < RPT; ++t) {
-                q_next[t] = t0[part * RPT + t];
-                k_next[t] = t0[DP + part * RPT + t];
-                g_next[t] = t0[2 * DP + part * RPT + t];
+                q_next[t] = t0[t * DELTA_LANES + part];
+                k_next[t] = t0[DP + t * DELTA_LANES + part];
+                g_next[t] = t0[2 * DP + t * DELTA_LANES + part];
             }
             b_next = t0[3 * DP];
             v_next = t0[3 * DP + 4 + local];
         };
         fetch(0);
         for (int token = 0; token < tokens; ++token) {
-            float q_now[RPT], k_now[RPT];
+            // The chain from token to token is: decay, the sum over key channels, the write. The read-out
+            // o = (S' + k u^T)^T q = S'^T q + u (k . q) with S' = diag(g) S is formed beside it from sums
+            // that do not wait for u: all three sums of a token travel through the lanes together.
+            float k_now[RPT];
             const float b = b_next, v = v_next;
-            float seen = 0.0f;
+            float seen = 0.0f, read_before = 0.0f, kq = 0.0f;
 #pragma unroll
             for (int t = 0; t < RPT; ++t) {
-                q_now[t] = q_next[t];
                 k_now[t] = k_next[t];
                 S[t] *= g_next[t];
                 seen = fmaf(S[t], k_now[t], seen);
+                read_before = fmaf(S[t], q_next[t], read_before);
+                kq = fmaf(k_now[t], q_next[t], kq);
             }
             fetch(token + 1 < DELTA_CHUNK ? token + 1 : token);      // (behind the chunk's last token: read again, not used)
             seen = delta_row_sum(seen);
+            read_before = delta_row_sum(read_before);
+            kq = delta_row_sum(kq);
             const float u = b * (v - seen);
-            float read = 0.0f;
 #pragma unroll
-            for (int t = 0; t < RPT; ++t) {
-                S[t] = fmaf(k_now[t], u, S[t]);
-                read = fmaf(S[t], q_now[t], read);
-            }
-            read = delta_row_sum(read);
-            if (part == 0) results[token * DELTA_COLUMNS + local] = read;
+            for (int t = 0; t < RPT; ++t) S[t] = fmaf(k_now[t], u, S[t]);
+            if (part == 0) results[token * DELTA_COLUMNS + local] = fmaf(u, kq, read_before);
         }
         __syncthreads();
         // the chunk's read-outs leave together: a token's 16 columns side by side
@@ -318,7 +320,7 @@ __global__ __launch_bounds__(256) void gated_delta_rule_kernel(
     if (live) {
 #pragma unroll
         for (int t = 0; t < RPT; ++t) {
-            const int i = part * RPT + t;
+            const int i = t * DELTA_LANES + part;
             if (i < dim) mine[i] = S[t];
         }
     }

@@ -69,12 +69,12 @@ CONFIG_Z = {
 }
 
 # W: wide enough that a prompt of some hundred tokens goes through the tiled prompt products and the
-# matrix-core attention (keys of 64, values of 128 channels and the other way round), with widths of
+# matrix-core attention (keys of 64 and values of 128 channels in one layer, the reverse in the other), with widths of
 # the joined operands that are no multiple of their tiles.
 CONFIG_W = {
     "architecture": "Koketar", "vocab": 1000, "width": 512, "norm": {"eps": 1e-5}, "residual_mult": 0.4, "logit_softcap": 20.0,
     "layers": [
-        _layer(_left(8, 2, 64, 128, 150, 32, 100000.0, 8.0, 0.125), _right(6, 3, 48, 80, 4, 24, 40), 0.8, 0.5, 1344, 1.0),
+        _layer(_left(8, 2, 64, 128, 150, 48, 100000.0, 4.0, 0.11), _right(6, 3, 48, 80, 4, 24, 40), 0.9, 0.6, 1344, 1.5),
         _layer(_left(4, 4, 128, 64, 90, 128, 100000.0, None, 0.09), _right(4, 4, 128, 128, 3, 16, 16), 1.0, 1.0, 1024, 2.0),
     ],
 }

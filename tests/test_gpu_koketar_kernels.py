@@ -246,7 +246,7 @@ def test_clamped_gated_unit_behind_its_product(rows):
     split-K product up to 64); more rows: float32 sums and the unit's own kernel. All against the plain formula."""
     from flyweight_amd.parts.linear import Linear
     rng = np.random.default_rng(rows)
-    hidden, inter, limit = 256, 384, 0.9
+    hidden, inter, limit = 320, 448, 0.9
     a = torch.from_numpy(rng.normal(size=(rows, hidden))).to(torch.bfloat16).cuda()
     w = torch.from_numpy(rng.normal(size=(2 * inter, hidden)) / 8).to(torch.bfloat16).cuda()
     got = Linear(w).clamped_glu(a, limit, 1.702, 1.0).float().cpu().numpy()
