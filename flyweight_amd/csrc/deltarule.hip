@@ -220,7 +220,7 @@ __global__ __launch_bounds__(256) void gated_delta_rule_kernel(
     for (int i = 0; i < PIECES; ++i) {
         const int item = threadIdx.x + 256 * i;
         const int token = item / per_token, f = (item % per_token) * 4;
-        piece_token[i] = token < DELTA_CHUNK ? token : DELTA_CHUNK;
+        piece_token[i] = token < DELTA_CHUNK ? token : DELTA_CHUNK;       // DELTA_CHUNK: this thread has no such piece
         int from, to;
         if (f < 3 * d4) {
             from = f;
@@ -232,7 +232,7 @@ __global__ __launch_bounds__(256) void gated_delta_rule_kernel(
             from = 3 * d4 + 4 + block * DELTA_COLUMNS + (f - 3 * d4 - 4);
             to = 3 * DP + 4 + (f - 3 * d4 - 4);
         }
-        piece_from[i] = from;
+        piece_from[i] = token < DELTA_CHUNK ? from : 0;
         piece_to[i] = (token < DELTA_CHUNK ? token : 0) * TOKEN + to;
     }
     const int staged_tokens = count < DELTA_CHUNK ? count : DELTA_CHUNK;     // a decode step stages one token
@@ -240,12 +240,16 @@ __global__ __launch_bounds__(256) void gated_delta_rule_kernel(
     const float* source = records + ((size_t)first * heads + head) * record;
     const size_t token_stride = (size_t)heads * record;
     f32x4 held[PIECES];
+    // Loads are unconditional (a piece past the chunk's end is read from a valid place again and never
+    // used): behind a branch the compiler would wait for each load at once, and the next chunk would
+    // not travel while this one is worked on.
     auto ask = [&](int base) {
-        const int tokens = count - base < DELTA_CHUNK ? count - base : DELTA_CHUNK;
+        const int last = (count - base < DELTA_CHUNK ? count - base : DELTA_CHUNK) - 1;
 #pragma unroll
-        for (int i = 0; i < PIECES; ++i)
-            if (piece_token[i] < tokens)
-                held[i] = *reinterpret_cast<const f32x4*>(source + (size_t)(base + piece_token[i]) * token_stride + piece_from[i]);
+        for (int i = 0; i < PIECES; ++i) {
+            const int token = piece_token[i] < last ? piece_token[i] : last;
+            held[i] = *reinterpret_cast<const f32x4*>(source + (size_t)(base + token) * token_stride + piece_from[i]);
+        }
     };
     auto put = [&](int base) {
         const int tokens = count - base < DELTA_CHUNK ? count - base : DELTA_CHUNK;

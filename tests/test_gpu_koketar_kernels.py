@@ -28,11 +28,13 @@ def record_layout(dim, vdim):
     return {"q": 0, "k": d4, "g": 2 * d4, "beta": 3 * d4, "v": 3 * d4 + 4, "floats": 3 * d4 + 4 + v4}
 
 
+@pytest.mark.parametrize("lengths,slots_of", [([37, 1, 18], [2, 0, 3]), ([150], [4]), ([70, 90], [1, 0])])
 @pytest.mark.parametrize("heads,kv_heads,dim,vdim", [(3, 1, 20, 70), (2, 2, 64, 64), (4, 2, 8, 5), (1, 1, 130, 129), (2, 1, 256, 16)])
-def test_recurrence_over_segments_with_carried_state(heads, kv_heads, dim, vdim):
+def test_recurrence_over_segments_with_carried_state(heads, kv_heads, dim, vdim, lengths, slots_of):
+    """Short segments and single rows (a column of the state over sixteen lanes) and long ones of one or
+    two sequences (over a whole wave), each from a state that is not zero."""
     from flyweight_amd.kernels import ops
     rng = np.random.default_rng(dim + vdim)
-    lengths, slots_of = [37, 1, 18], [2, 0, 3]
     rows = sum(lengths)
     q = plain.unit(rng.normal(size=(rows, kv_heads, dim))) * dim ** -0.5
     k = plain.unit(rng.normal(size=(rows, kv_heads, dim)))
