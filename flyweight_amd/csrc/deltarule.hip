@@ -310,16 +310,16 @@ __global__ __launch_bounds__(256) void gated_delta_rule_kernel(
             for (int t = 0; t < RPT; ++t) S[t] = fmaf(k_now[t], u, S[t]);
             if (part == 0) results[token * DELTA_COLUMNS + local] = fmaf(u, kq, read_before);
         }
-        __syncthreads();
+        // (barriers that order LDS traffic only: the next chunk's loads stay in flight across them)
+        fw_lds_barrier();
         // the chunk's read-outs leave together: a token's 16 columns side by side
         {
             const int token = threadIdx.x / DELTA_COLUMNS, c = threadIdx.x % DELTA_COLUMNS;
             if (token < tokens && block * DELTA_COLUMNS + c < vdim)
                 out[((size_t)first + base + token) * heads * vdim + head * vdim + block * DELTA_COLUMNS + c] = results[threadIdx.x];
         }
-        __syncthreads();
         if (more) put(base + DELTA_CHUNK);
-        __syncthreads();
+        fw_lds_barrier();
     }
     if (live) {
 #pragma unroll
