@@ -2,8 +2,9 @@
 design's equations. It shares no code with the package: the tests hold the engine against it.
 
 Notation: T tokens, D model width; a weight W is stored [out, in] and applied as x @ W.T.
-Every function takes whole sequences (position 0 first) except ``delta_rule_step`` and the
-``Stream`` class, which carry a request's state from token to token.
+Every function takes whole sequences (position 0 first) except ``delta_rule_step``, which takes
+one token and the state before it, and ``delta_inputs`` / ``causal_conv``, which may be told what
+came before.
 """
 
 from __future__ import annotations
@@ -236,7 +237,10 @@ def random_weights(config: dict, seed: int) -> Dict[str, np.ndarray]:
         elif leaf == "dt_bias":
             value = rng.uniform(-3.0, 0.0, shape)
         elif name == "embed":
-            value = rng.normal(0.0, 1.0, shape)
+            # small beside what the layers add: a token's own embedding must not decide the logits of the
+            # tied head (greedy generation would repeat the last token whatever the mixers do), and the
+            # logits stay below a soft cap's flat part
+            value = rng.normal(0.0, 0.2, shape)
         else:
             value = rng.normal(0.0, 1.0 / math.sqrt(shape[-1]), shape)
         out[name] = value
