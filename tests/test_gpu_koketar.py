@@ -274,3 +274,24 @@ def test_command_line(models, capsys, tmp_path):
     assert main(["generate", str(tmp_path / "drawn"), "--tokens", "1,2,3", "--max-tokens", "4", "--temperature", "0",
                  "--ignore-eos", "--context", "128"]) == 0
     assert len(capsys.readouterr().out.split()) == 4
+
+
+def test_serving_more_requests_than_slots_on_few_pages(models):
+    """Seven requests through three slots and four pages a group, several decode steps per turn on
+    the device: requests wait for a slot, slots and pages are handed on, recorded decode steps are
+    replayed at changing batch sizes. The tokens are the plain model's (float32)."""
+    import flyweight_amd
+    loaded = models("Y", "float32")
+    vocab = loaded.config["vocab"]
+    prompts = [random_tokens(vocab, n, seed=60 + n) for n in (90, 3, 150, 64, 65, 1, 120)]
+    new = [9, 14, 6, 11, 5, 16, 8]
+    want = [plain.greedy(loaded.config, loaded.weights, p, n) for p, n in zip(prompts, new)]
+    assert len({tuple(w) for w in want}) == len(want) and all(len(set(w)) > 2 for w in want if len(w) > 6)    # no trivial outputs
+    with flyweight_amd.Runtime(flyweight_amd.Model(loaded.folder, dtype="float32"), context_limit=192, parallel_sequences=3,
+                               num_pages=4, prefill_rows=48, max_batch_tokens=56, decode_steps_per_turn=4) as runtime:
+        tasks = [runtime.task_submit(p, n) for p, n in zip(prompts, new)]
+        result = runtime.run()
+        assert runtime.info["live_requests"] == 0
+        runtime.stepper.cache.check_invariants()
+    for task, expected in zip(tasks, want):
+        assert result[task] == expected
