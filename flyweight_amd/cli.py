@@ -102,6 +102,7 @@ def build_parser() -> argparse.ArgumentParser:
     replay.add_argument("--dtype", required=True, choices=("bfloat16", "float32"))
     replay.add_argument("--out", required=True, metavar="DIR")
     replay.add_argument("--max-tokens", required=True, type=int, metavar="N")
+    replay.add_argument("--max-requests", type=int, default=4, metavar="N", help="state slots: the most requests live at once")
     return parser
 
 
@@ -223,7 +224,7 @@ def main(argv: Optional[List[str]] = None) -> int:
             return _random_weights(args)
         if args.command == "replay":
             from .engine.trace import replay
-            return replay(args.model, args.dtype, args.out, args.max_tokens, sys.stdin, sys.stdout)
+            return replay(args.model, args.dtype, args.out, args.max_tokens, sys.stdin, sys.stdout, max_requests=args.max_requests)
     except (ValueError, RuntimeError, OSError) as error:
         print(f"flyweight-amd: {error}", file=sys.stderr)
         return 1

@@ -22,7 +22,7 @@ __global__ __launch_bounds__(64) void qk_norm_rope_kv_write_kernel(
     const float* __restrict__ k_norm_weight, float eps, const float* __restrict__ cos_table,
     const float* __restrict__ sin_table, int rotary_dim, T* __restrict__ k_pages, T* __restrict__ v_pages,
     const int32_t* __restrict__ block_table, int table_stride, const int32_t* __restrict__ row_seg,
-    const int32_t* __restrict__ row_pos, int num_heads, int num_kv_heads, int head_dim, int v_dim) {
+    const int32_t* __restrict__ row_pos, int num_heads, int num_kv_heads, int head_dim, int v_dim, int interleaved) {
     __shared__ float normed[ATTN_MAX_HEAD_DIM];
     const int row = blockIdx.x;
     const int vec = blockIdx.y;
@@ -64,11 +64,13 @@ __global__ __launch_bounds__(64) void qk_norm_rope_kv_write_kernel(
     for (int d = lane; d < head_dim; d += 64) {
         float value = normed[d];
         if (d < rotary_dim) {
-            const int pair = d < half ? d : d - half;
-            const float other = normed[d < half ? d + half : d - half];
+            // the pair's first channel turns as u cos - v sin, its second as v cos + u sin
+            const bool is_first = interleaved ? (d & 1) == 0 : d < half;
+            const int pair = interleaved ? d >> 1 : (d < half ? d : d - half);
+            const float other = normed[interleaved ? d ^ 1 : (d < half ? d + half : d - half)];
             const float c = cos_table[(size_t)row * half + pair];
             const float s = sin_table[(size_t)row * half + pair];
-            value = d < half ? value * c - other * s : value * c + other * s;
+            value = is_first ? value * c - other * s : value * c + other * s;
         }
         store_from_float(dest, d, value);
     }
@@ -87,7 +89,7 @@ __global__ __launch_bounds__(64) void qk_norm_rope_kv_write_rows_kernel(
     const float* __restrict__ k_norm_weight, float eps, const float* __restrict__ cos_table,
     const float* __restrict__ sin_table, int rotary_dim, T* __restrict__ k_pages, T* __restrict__ v_pages,
     const int32_t* __restrict__ block_table, int table_stride, const int32_t* __restrict__ row_seg,
-    const int32_t* __restrict__ row_pos, int num_heads, int num_kv_heads, int head_dim, int rows) {
+    const int32_t* __restrict__ row_pos, int num_heads, int num_kv_heads, int head_dim, int rows, int interleaved) {
     const int r0 = blockIdx.x * QK_ROWS;
     const int vec = blockIdx.y;
     const int lane = threadIdx.x;
@@ -97,7 +99,9 @@ __global__ __launch_bounds__(64) void qk_norm_rope_kv_write_rows_kernel(
     const float* weight = is_value ? nullptr : (is_query ? q_norm_weight : k_norm_weight);
     const int half = rotary_dim / 2;
     const bool turned = !is_value && lane < rotary_dim;
-    const int pair = lane < half ? lane : lane - half;
+    const bool is_first = interleaved ? (lane & 1) == 0 : lane < half;
+    const int pair = interleaved ? lane >> 1 : (lane < half ? lane : lane - half);
+    const int partner = interleaved ? lane ^ 1 : (lane < half ? lane + half : lane - half);
     int row_of[QK_ROWS], pos[QK_ROWS], page[QK_ROWS];
     float v[QK_ROWS], c[QK_ROWS], sn[QK_ROWS];
 #pragma unroll
@@ -153,8 +157,8 @@ __global__ __launch_bounds__(64) void qk_norm_rope_kv_write_rows_kernel(
             const float inv = rsqrtf(sum / (float)head_dim + eps);
             value = value * inv * w;
         }
-        const float other = __shfl(value, lane < half ? lane + half : lane - half, 64);
-        if (lane < rotary_dim) value = lane < half ? value * c[i] - other * sn[i] : value * c[i] + other * sn[i];
+        const float other = __shfl(value, partner & 63, 64);
+        if (lane < rotary_dim) value = is_first ? value * c[i] - other * sn[i] : value * c[i] + other * sn[i];
         T* dest = is_query ? q_out + ((size_t)row_of[i] * num_heads + vec) * head_dim
                            : k_pages + (((size_t)page[i] * num_kv_heads + (vec - num_heads)) * ATTN_PAGE + slot) * head_dim;
         if (active) store_from_float(dest, lane, value);
@@ -166,7 +170,8 @@ extern "C" int fw_qk_norm_rope_kv_write(const void* qkv, int in_dtype, void* q_o
                                         const float* sin_table, int rotary_dim, void* k_pages, void* v_pages,
                                         const int32_t* block_table, int table_stride, const int32_t* row_seg,
                                         const int32_t* row_pos, int rows, int num_heads, int num_kv_heads,
-                                        int head_dim, int v_dim, int page_size, int num_pages, int write_kv, void* stream) {
+                                        int head_dim, int v_dim, int page_size, int num_pages, int write_kv, int interleaved,
+                                        void* stream) {
     FW_REQUIRE(rows >= 0 && num_heads > 0 && num_kv_heads > 0, "qk_norm_rope: bad sizes rows=%d heads=%d kv_heads=%d", rows, num_heads, num_kv_heads);
     FW_REQUIRE(head_dim > 0 && head_dim <= ATTN_MAX_HEAD_DIM, "qk_norm_rope: head_dim %d outside 1..%d", head_dim, ATTN_MAX_HEAD_DIM);
     FW_REQUIRE(v_dim > 0 && v_dim <= ATTN_MAX_HEAD_DIM, "qk_norm_rope: value size %d outside 1..%d", v_dim, ATTN_MAX_HEAD_DIM);
@@ -186,7 +191,7 @@ extern "C" int fw_qk_norm_rope_kv_write(const void* qkv, int in_dtype, void* q_o
 #define FW_QK_ROWS_LAUNCH(TI, T)                                                                                     \
     qk_norm_rope_kv_write_rows_kernel<TI, T><<<by_rows, 64, 0, s>>>(                                                 \
         (const TI*)qkv, (T*)q_out, q_norm_weight, k_norm_weight, eps, cos_table, sin_table, rotary_dim, (T*)k_pages, \
-        (T*)v_pages, block_table, table_stride, row_seg, row_pos, num_heads, num_kv_heads, head_dim, rows)
+        (T*)v_pages, block_table, table_stride, row_seg, row_pos, num_heads, num_kv_heads, head_dim, rows, interleaved)
         if (in_dtype == FW_F32 && dtype == FW_F32) FW_QK_ROWS_LAUNCH(float, float);
         else if (in_dtype == FW_F32 && dtype == FW_BF16) FW_QK_ROWS_LAUNCH(float, bf16_t);
         else if (in_dtype == FW_BF16 && dtype == FW_BF16) FW_QK_ROWS_LAUNCH(bf16_t, bf16_t);
@@ -198,7 +203,7 @@ extern "C" int fw_qk_norm_rope_kv_write(const void* qkv, int in_dtype, void* q_o
 #define FW_QK_LAUNCH(TI, T)                                                                                          \
     qk_norm_rope_kv_write_kernel<TI, T><<<grid, 64, 0, s>>>(                                                         \
         (const TI*)qkv, (T*)q_out, q_norm_weight, k_norm_weight, eps, cos_table, sin_table, rotary_dim, (T*)k_pages, \
-        (T*)v_pages, block_table, table_stride, row_seg, row_pos, num_heads, num_kv_heads, head_dim, v_dim)
+        (T*)v_pages, block_table, table_stride, row_seg, row_pos, num_heads, num_kv_heads, head_dim, v_dim, interleaved)
     if (in_dtype == FW_F32 && dtype == FW_F32) FW_QK_LAUNCH(float, float);
     else if (in_dtype == FW_F32 && dtype == FW_BF16) FW_QK_LAUNCH(float, bf16_t);
     else if (in_dtype == FW_BF16 && dtype == FW_BF16) FW_QK_LAUNCH(bf16_t, bf16_t);
@@ -217,7 +222,8 @@ template <typename T>
 __global__ __launch_bounds__(64) void attention_generic_kernel(
     const T* __restrict__ q, T* __restrict__ out, const T* __restrict__ k_pages, const T* __restrict__ v_pages,
     const int32_t* __restrict__ block_table, int table_stride, const int32_t* __restrict__ row_seg,
-    const int32_t* __restrict__ row_pos, int num_heads, int num_kv_heads, int head_dim, int v_dim, float scale, int window) {
+    const int32_t* __restrict__ row_pos, int num_heads, int num_kv_heads, int head_dim, int v_dim, float scale, int window,
+    int chunk, float softcap) {
     __shared__ float qs[ATTN_MAX_HEAD_DIM];
     __shared__ float ps[ATTN_PAGE];
     const int row = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
@@ -227,7 +233,7 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
     const T* query = q + ((size_t)row * num_heads + head) * head_dim;
     for (int d = lane; d < head_dim; d += 64) qs[d] = load_as_float(query, d);
     __syncthreads();
-    const int first = window > 0 ? (pos - window + 1 > 0 ? pos - window + 1 : 0) : 0;
+    const int first = fw_first_visible(pos, window, chunk);
     float running_max = -INFINITY, running_sum = 0.0f;
     float acc[ATTN_MAX_HEAD_DIM / 64] = {};
     for (int tile = first / ATTN_PAGE; tile <= pos / ATTN_PAGE; ++tile) {
@@ -240,6 +246,7 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
             float dot = 0.0f;
             for (int d = 0; d < head_dim; ++d) dot = fmaf(qs[d], load_as_float(key, d), dot);
             score = dot * scale;
+            if (softcap > 0.0f) score = softcap * tanhf(score / softcap);
         }
         const float new_max = fmaxf(running_max, wave_max(score));
         const float p = valid ? expf(score - new_max) : 0.0f;
@@ -273,8 +280,9 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
 extern "C" int fw_attention_generic(const void* q, void* out, int dtype, const void* k_pages,
                                     const void* v_pages, const int32_t* block_table, int table_stride,
                                     const int32_t* row_seg, const int32_t* row_pos, int rows, int num_heads,
-                                    int num_kv_heads, int head_dim, int v_dim, float scale, int window, int page_size,
-                                    int num_pages, void* stream) {
+                                    int num_kv_heads, int head_dim, int v_dim, float scale, int window, int chunk,
+                                    float softcap, int page_size, int num_pages, void* stream) {
+    FW_REQUIRE(chunk >= 0 && softcap >= 0.0f, "attention: chunk %d and soft cap %g must not be negative", chunk, (double)softcap);
     FW_REQUIRE(rows >= 0 && num_heads > 0 && num_kv_heads > 0 && num_heads % num_kv_heads == 0,
                "attention: heads %d must be a positive multiple of kv heads %d", num_heads, num_kv_heads);
     FW_REQUIRE(head_dim > 0 && head_dim <= ATTN_MAX_HEAD_DIM, "attention: head_dim %d outside 1..%d", head_dim, ATTN_MAX_HEAD_DIM);
@@ -288,11 +296,11 @@ extern "C" int fw_attention_generic(const void* q, void* out, int dtype, const v
     if (dtype == FW_F32)
         attention_generic_kernel<float><<<grid, 64, 0, (hipStream_t)stream>>>(
             (const float*)q, (float*)out, (const float*)k_pages, (const float*)v_pages, block_table, table_stride,
-            row_seg, row_pos, num_heads, num_kv_heads, head_dim, v_dim, scale, window);
+            row_seg, row_pos, num_heads, num_kv_heads, head_dim, v_dim, scale, window, chunk, softcap);
     else if (dtype == FW_BF16)
         attention_generic_kernel<bf16_t><<<grid, 64, 0, (hipStream_t)stream>>>(
             (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)k_pages, (const bf16_t*)v_pages, block_table, table_stride,
-            row_seg, row_pos, num_heads, num_kv_heads, head_dim, v_dim, scale, window);
+            row_seg, row_pos, num_heads, num_kv_heads, head_dim, v_dim, scale, window, chunk, softcap);
     else
         FW_REQUIRE(false, "attention: unknown dtype %d", dtype);
     FW_LAUNCH_CHECK("attention_generic");

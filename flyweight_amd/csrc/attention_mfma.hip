@@ -74,7 +74,8 @@ struct Columns {
 template <int HD, int NH, bool CLEAN_V, bool K_PADDED, bool EARLY_V = false>
 __device__ __forceinline__ void attend_page(Columns<HD> (&c)[NH], const uint16_t* __restrict__ k_page,
                                             const uint16_t* __restrict__ v_page, int head_dim, int v_dim, float scale_log2,
-                                            int lo, int hi, int last_written, int k_stride, int v_stride) {
+                                            int lo, int hi, int last_written, int k_stride, int v_stride,
+                                            float cap = 0.0f, float cap_scale = 0.0f) {
     const int lane = threadIdx.x & 63;
     const int i16 = lane & 15, g = lane >> 4;
     // all key loads of the page are issued before the first product
@@ -117,6 +118,21 @@ __device__ __forceinline__ void attend_page(Columns<HD> (&c)[NH], const uint16_t
             for (int dc = 0; dc < HD / 32; ++dc)
                 s[h][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[kt][dc], c[h].q[dc], s[h][kt], 0, 0, 0);
         }
+    // A soft cap on the scores: s <- cap * tanh(s * scale / cap) (cap_scale = scale / cap; the caller then
+    // passes log2(e) as the exponent's scale). tanh(x) = 1 - 2 / (1 + e^2x): exact at both ends, where
+    // e^2x is 0 or infinite; the hardware's 2^x and reciprocal leave the scores to about 1e-6 of the cap.
+    if (cap > 0.0f) {
+        const float twice = 2.0f * cap_scale * 1.4426950408889634f;
+#pragma unroll
+        for (int h = 0; h < NH; ++h)
+#pragma unroll
+            for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const float e = __builtin_amdgcn_exp2f(s[h][kt][r] * twice);
+                    s[h][kt][r] = cap - 2.0f * cap * __builtin_amdgcn_rcpf(1.0f + e);
+                }
+    }
     const bool full = __all(lo <= 0 && hi >= PAGE - 1) && last_written >= PAGE - 1;
     if (!full) {
 #pragma unroll
@@ -264,7 +280,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((HD <= 64 &
     const uint16_t* __restrict__ q, uint16_t* __restrict__ out, const uint16_t* __restrict__ k_pages,
     const uint16_t* __restrict__ v_pages, const int32_t* __restrict__ block_table, int table_stride,
     const int32_t* __restrict__ tile_seg, const int32_t* __restrict__ tile_row0, const int32_t* __restrict__ seg_row0,
-    const int32_t* __restrict__ row_pos, int num_heads, int num_kv_heads, int head_dim, int v_dim, float scale_log2, int window) {
+    const int32_t* __restrict__ row_pos, int num_heads, int num_kv_heads, int head_dim, int v_dim, float scale_log2, int window,
+    int chunk, float cap, float cap_scale) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     // a key's row in LDS holds HD channels, those past head_dim zero: every lane loads its operand
     constexpr int k_stride = HD + KV_PAD;
@@ -295,8 +312,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((HD <= 64 &
     const int my_pos = row_pos[my_row];
     const int wave_hi = rows > 0 ? row_pos[row0 + rows - 1] : -1;       // last position of this wave
     const int pos_lo = row_pos[tile_first_row], pos_hi = row_pos[tile_first_row + tile_rows - 1];
-    const int my_first = window > 0 && my_pos - window + 1 > 0 ? my_pos - window + 1 : 0;
-    const int tile_first = window > 0 && pos_lo - window + 1 > 0 ? pos_lo - window + 1 : 0;
+    const int my_first = fw_first_visible(my_pos, window, chunk);
+    const int tile_first = fw_first_visible(pos_lo, window, chunk);      // the first key never falls as the position rises
 
     // a head past the end of the group computes along on zeros and is not stored
     Columns<HD> c[NH];
@@ -368,7 +385,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((HD <= 64 &
             // a lane without a row computes along with the bounds of the tile's first row (nothing of
             // it is stored): a page that is whole for the rows is then whole for the wave
             attend_page<HD, NH, false, true>(c, kt, kt + k_elems, head_dim, v_dim, scale_log2, my_first - base, my_pos - base, pos_hi - base,
-                            k_stride, v_stride);
+                            k_stride, v_stride, cap, cap_scale);
         }
     };
 
@@ -430,6 +447,7 @@ struct FusedProjections {
     const float* sin_table;
     int rotary_dim;
     int write_kv;                   // 0: another execution of the layer has stored this step's keys and values already
+    int interleaved;                // 0: channel i turns with channel i + rotary_dim / 2; 1: channel 2i with channel 2i + 1
 };
 
 // One head-vector of head_dim channels by one wave: optional RMS norm, then the half-split rotation
@@ -438,7 +456,7 @@ struct FusedProjections {
 template <typename Store>
 __device__ __forceinline__ void norm_rotate_vector(const float* __restrict__ source, const float* __restrict__ weight, float eps,
                                                    const float* __restrict__ cos_row, const float* __restrict__ sin_row,
-                                                   int rotary_dim, int head_dim, float* scratch, Store store) {
+                                                   int rotary_dim, int head_dim, float* scratch, Store store, int interleaved = 0) {
     const int lane = threadIdx.x & 63;
     float inv = 1.0f;
     if (weight) {
@@ -461,10 +479,11 @@ __device__ __forceinline__ void norm_rotate_vector(const float* __restrict__ sou
     for (int d = lane; d < head_dim; d += 64) {
         float value = scratch[d];
         if (d < rotary_dim) {
-            const int pair = d < half ? d : d - half;
-            const float other = scratch[d < half ? d + half : d - half];
+            const bool is_first = interleaved ? (d & 1) == 0 : d < half;
+            const int pair = interleaved ? d >> 1 : (d < half ? d : d - half);
+            const float other = scratch[interleaved ? d ^ 1 : (d < half ? d + half : d - half)];
             const float c = cos_row[pair], s = sin_row[pair];
-            value = d < half ? value * c - other * s : value * c + other * s;
+            value = is_first ? value * c - other * s : value * c + other * s;
         }
         store(d, value);
     }
@@ -475,7 +494,8 @@ __global__ __launch_bounds__(64 * SPLIT_PAGES) __attribute__((amdgpu_waves_per_e
     const uint16_t* __restrict__ q, uint16_t* __restrict__ out, float* partial, int* tickets,
     uint16_t* k_pages, uint16_t* v_pages, const int32_t* __restrict__ block_table, int table_stride,
     const int32_t* __restrict__ row_seg, const int32_t* __restrict__ row_pos, int num_heads, int num_kv_heads,
-    int head_dim, int v_dim, float scale_log2, int window, int max_splits, const int32_t* __restrict__ decode_work, const FusedProjections fused) {
+    int head_dim, int v_dim, float scale_log2, int window, int chunk, float cap, float cap_scale, int max_splits,
+    const int32_t* __restrict__ decode_work, const FusedProjections fused) {
     __shared__ f32x4 shared_o[SPLIT_PAGES][HD / 16][64];
     __shared__ float shared_m[SPLIT_PAGES][16], shared_l[SPLIT_PAGES][16];
     __shared__ int ticket_shared;
@@ -488,7 +508,7 @@ __global__ __launch_bounds__(64 * SPLIT_PAGES) __attribute__((amdgpu_waves_per_e
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, col = lane & 15, g = lane >> 4;
     const int pos = row_pos[row];
     const int segment = row_seg[row];       // asked for together with the position, not behind the branch below
-    const int first = window > 0 && pos - window + 1 > 0 ? pos - window + 1 : 0;
+    const int first = fw_first_visible(pos, window, chunk);
     // Splits are counted from the first page that holds a visible key; a split is `rounds` runs of
     // SPLIT_PAGES pages. One run each serves while the step's runs (decode_work: over all its rows;
     // times the kv heads and head tiles) are no more than about two workgroups per compute unit;
@@ -529,12 +549,12 @@ __global__ __launch_bounds__(64 * SPLIT_PAGES) __attribute__((amdgpu_waves_per_e
                 uint16_t* dest = fused_q[v];
                 norm_rotate_vector(projections + (size_t)(kvh * group + head_tile * 16 + v) * head_dim, fused.q_norm_weight, fused.eps,
                                    cos_row, sin_row, fused.rotary_dim, head_dim, fused_scratch[wave],
-                                   [&](int d, float value) { dest[d] = float_to_bf16_bits(value); });
+                                   [&](int d, float value) { dest[d] = float_to_bf16_bits(value); }, fused.interleaved);
             } else if (v == columns) {
                 uint16_t* dest = k_pages + (((size_t)own_page * num_kv_heads + kvh) * PAGE + slot) * head_dim;
                 norm_rotate_vector(projections + (size_t)(num_heads + kvh) * head_dim, fused.k_norm_weight, fused.eps, cos_row, sin_row,
                                    fused.rotary_dim, head_dim, fused_scratch[wave],
-                                   [&](int d, float value) { dest[d] = float_to_bf16_bits(value); });
+                                   [&](int d, float value) { dest[d] = float_to_bf16_bits(value); }, fused.interleaved);
             } else {
                 const float* value = projections + (size_t)(num_heads + num_kv_heads) * head_dim + (size_t)kvh * v_dim;
                 uint16_t* dest = v_pages + ((size_t)own_page * num_kv_heads + kvh) * v_dim * PAGE + slot;
@@ -556,7 +576,7 @@ __global__ __launch_bounds__(64 * SPLIT_PAGES) __attribute__((amdgpu_waves_per_e
         const int base = block * PAGE;
         // a lane without a head computes along (q = 0, nothing of it is stored)
         attend_page<HD, 1, true, false, (HD <= 128)>(columns_of_wave, k_pages + at * head_dim, v_pages + at * v_dim, head_dim, v_dim, scale_log2, first - base, pos - base, pos - base,
-                        head_dim, PAGE);
+                        head_dim, PAGE, cap, cap_scale);
     }
     const float l = fw_quad_sum(c.l);
 #pragma unroll
@@ -656,8 +676,25 @@ __global__ __launch_bounds__(64 * SPLIT_PAGES) __attribute__((amdgpu_waves_per_e
 
 static const float LOG2E = 1.4426950408889634f;
 
+// What the mask and the soft cap hand to the kernels: with a cap the scores are scaled and capped before
+// the softmax, whose exponent then takes log2(e) alone.
+struct ScoreRule {
+    float scale_log2, cap, cap_scale;
+};
+static ScoreRule score_rule(float scale, float softcap) {
+    if (softcap > 0.0f) return ScoreRule{LOG2E, softcap, scale / softcap};
+    return ScoreRule{scale * LOG2E, 0.0f, 0.0f};
+}
+// the most keys a row can see where a window or a chunk bounds them (0: all)
+static int visible_span(int window, int chunk) {
+    int span = window;
+    if (chunk > 0 && (span == 0 || chunk < span)) span = chunk;
+    return span;
+}
+
 static int check_common(const char* name, int rows, int num_heads, int num_kv_heads, int head_dim, int v_dim, int page_size,
-                        int window, int num_pages, int table_stride) {
+                        int window, int num_pages, int table_stride, int chunk = 0, float softcap = 0.0f) {
+    FW_REQUIRE(chunk >= 0 && softcap >= 0.0f, "%s: chunk %d and soft cap %g must not be negative", name, chunk, (double)softcap);
     FW_REQUIRE(rows >= 0 && num_heads > 0 && num_kv_heads > 0 && num_heads % num_kv_heads == 0,
                "%s: heads %d must be a positive multiple of kv heads %d", name, num_heads, num_kv_heads);
     FW_REQUIRE(head_dim >= 16 && head_dim <= 256 && head_dim % 16 == 0, "%s: head_dim %d must be a multiple of 16 in 16..256", name, head_dim);
@@ -688,9 +725,10 @@ extern "C" int fw_attention_prefill(const void* q, void* out, const void* k_page
                                     const int32_t* block_table, int table_stride, const int32_t* tile_seg,
                                     const int32_t* tile_row0, int tiles, const int32_t* seg_row0,
                                     const int32_t* row_pos, int rows, int num_heads, int num_kv_heads, int head_dim,
-                                    int v_dim, float scale, int window, int page_size, int num_pages, int heads_together,
-                                    void* stream) {
-    if (check_common("attention_prefill", rows, num_heads, num_kv_heads, head_dim, v_dim, page_size, window, num_pages, table_stride)) return -1;
+                                    int v_dim, float scale, int window, int chunk, float softcap, int page_size, int num_pages,
+                                    int heads_together, void* stream) {
+    if (check_common("attention_prefill", rows, num_heads, num_kv_heads, head_dim, v_dim, page_size, window, num_pages, table_stride, chunk, softcap)) return -1;
+    const ScoreRule rule = score_rule(scale, softcap);
     const int widest = head_dim > v_dim ? head_dim : v_dim;      // the template holds both
     FW_REQUIRE(tiles >= 0 && tiles <= rows && num_heads <= 65535, "attention_prefill: %d tiles for %d rows", tiles, rows);
     const int most_together = widest <= 64 ? 4 : 1;
@@ -716,7 +754,7 @@ extern "C" int fw_attention_prefill(const void* q, void* out, const void* k_page
         attention_prefill_kernel<HD, NH><<<grid, 256, lds_bytes, (hipStream_t)stream>>>(                            \
             (const uint16_t*)q, (uint16_t*)out, (const uint16_t*)k_pages, (const uint16_t*)v_pages, block_table,    \
             table_stride, tile_seg, tile_row0, seg_row0, row_pos, num_heads, num_kv_heads, head_dim, v_dim,        \
-            scale * LOG2E, window);                                                                                \
+            rule.scale_log2, window, chunk, rule.cap, rule.cap_scale);                                             \
     }
     if (widest <= 32) {
         if (heads_together == 4) LAUNCH(32, 4) else LAUNCH(32, 1)
@@ -733,8 +771,9 @@ extern "C" int fw_attention_prefill(const void* q, void* out, const void* k_page
 }
 
 static int decode_check(int max_splits, int max_context, int* tickets, int tickets_len, int table_stride, int rows, int num_heads,
-                        int num_kv_heads, int head_dim, int v_dim, int window, int page_size, int num_pages) {
-    if (check_common("attention_decode", rows, num_heads, num_kv_heads, head_dim, v_dim, page_size, window, num_pages, table_stride)) return -1;
+                        int num_kv_heads, int head_dim, int v_dim, int window, int page_size, int num_pages, int chunk, float softcap) {
+    if (check_common("attention_decode", rows, num_heads, num_kv_heads, head_dim, v_dim, page_size, window, num_pages, table_stride, chunk, softcap)) return -1;
+    window = visible_span(window, chunk);       // below: what bounds the pages a row's keys lie in
     FW_REQUIRE(max_splits >= 1 && max_splits <= 65535, "attention_decode: max_splits %d outside 1..65535", max_splits);
     FW_REQUIRE(max_context >= 1, "attention_decode: max_context must be positive");
     int blocks = (max_context + PAGE - 1) / PAGE;
@@ -752,9 +791,10 @@ static int decode_check(int max_splits, int max_context, int* tickets, int ticke
 
 static int decode_launch(const void* q, void* out, float* partial, int max_splits, const int32_t* decode_work, int* tickets, void* k_pages, void* v_pages,
                          const int32_t* block_table, int table_stride, const int32_t* row_seg, const int32_t* row_pos, int rows,
-                         int num_heads, int num_kv_heads, int head_dim, int v_dim, float scale, int window, const FusedProjections& fused,
-                         void* stream) {
+                         int num_heads, int num_kv_heads, int head_dim, int v_dim, float scale, int window, int chunk, float softcap,
+                         const FusedProjections& fused, void* stream) {
     if (rows == 0) return 0;
+    const ScoreRule rule = score_rule(scale, softcap);
     const int head_tiles = (num_heads / num_kv_heads + 15) / 16;
     dim3 grid(rows, num_kv_heads * head_tiles, max_splits);
 
@@ -762,11 +802,11 @@ static int decode_launch(const void* q, void* out, float* partial, int max_split
     if (fused.qkv)                                                                                                            \
         attention_decode_split_kernel<HD, true><<<grid, 64 * SPLIT_PAGES, 0, (hipStream_t)stream>>>(                          \
             (const uint16_t*)q, (uint16_t*)out, partial, tickets, (uint16_t*)k_pages, (uint16_t*)v_pages, block_table,        \
-            table_stride, row_seg, row_pos, num_heads, num_kv_heads, head_dim, v_dim, scale * LOG2E, window, max_splits, decode_work, fused); \
+            table_stride, row_seg, row_pos, num_heads, num_kv_heads, head_dim, v_dim, rule.scale_log2, window, chunk, rule.cap, rule.cap_scale, max_splits, decode_work, fused); \
     else                                                                                                                      \
         attention_decode_split_kernel<HD, false><<<grid, 64 * SPLIT_PAGES, 0, (hipStream_t)stream>>>(                         \
             (const uint16_t*)q, (uint16_t*)out, partial, tickets, (uint16_t*)k_pages, (uint16_t*)v_pages, block_table,        \
-            table_stride, row_seg, row_pos, num_heads, num_kv_heads, head_dim, v_dim, scale * LOG2E, window, max_splits, decode_work, fused)
+            table_stride, row_seg, row_pos, num_heads, num_kv_heads, head_dim, v_dim, rule.scale_log2, window, chunk, rule.cap, rule.cap_scale, max_splits, decode_work, fused)
     FW_BY_HEAD_DIM((head_dim > v_dim ? head_dim : v_dim), CALL);
 #undef CALL
     FW_LAUNCH_CHECK("attention_decode");
@@ -785,12 +825,12 @@ extern "C" int fw_attention_decode(const void* q, void* out, float* partial, int
                                    const int32_t* decode_work, int* tickets, int tickets_len, const void* k_pages,
                                    const void* v_pages, const int32_t* block_table, int table_stride,
                                    const int32_t* row_seg, const int32_t* row_pos, int rows, int num_heads,
-                                   int num_kv_heads, int head_dim, int v_dim, float scale, int window, int page_size,
-                                   int num_pages, void* stream) {
+                                   int num_kv_heads, int head_dim, int v_dim, float scale, int window, int chunk, float softcap,
+                                   int page_size, int num_pages, void* stream) {
     if (decode_check(max_splits, max_context, tickets, tickets_len, table_stride, rows, num_heads, num_kv_heads, head_dim, v_dim, window,
-                     page_size, num_pages)) return -1;
+                     page_size, num_pages, chunk, softcap)) return -1;
     return decode_launch(q, out, partial, max_splits, decode_work, tickets, const_cast<void*>(k_pages), const_cast<void*>(v_pages), block_table,
-                         table_stride, row_seg, row_pos, rows, num_heads, num_kv_heads, head_dim, v_dim, scale, window, FusedProjections{}, stream);
+                         table_stride, row_seg, row_pos, rows, num_heads, num_kv_heads, head_dim, v_dim, scale, window, chunk, softcap, FusedProjections{}, stream);
 }
 
 // fw_attention_decode with the work of fw_qk_norm_rope_kv_write in front of it, in the same kernel:
@@ -803,10 +843,10 @@ extern "C" int fw_attention_decode_fused(const float* qkv, const float* q_norm_w
                                          float* partial, int max_splits, int max_context, const int32_t* decode_work, int* tickets, int tickets_len,
                                          void* k_pages, void* v_pages, const int32_t* block_table, int table_stride,
                                          const int32_t* row_seg, const int32_t* row_pos, int rows, int num_heads,
-                                         int num_kv_heads, int head_dim, int v_dim, float scale, int window, int page_size, int num_pages,
-                                         void* stream) {
+                                         int num_kv_heads, int head_dim, int v_dim, float scale, int window, int chunk, float softcap,
+                                         int interleaved, int page_size, int num_pages, void* stream) {
     if (decode_check(max_splits, max_context, tickets, tickets_len, table_stride, rows, num_heads, num_kv_heads, head_dim, v_dim, window,
-                     page_size, num_pages)) return -1;
+                     page_size, num_pages, chunk, softcap)) return -1;
     FW_REQUIRE(qkv != nullptr, "attention_decode_fused: the projections are missing");
     FW_REQUIRE(rotary_dim >= 0 && rotary_dim <= head_dim && rotary_dim % 2 == 0, "attention_decode_fused: rotary_dim %d with head_dim %d",
                rotary_dim, head_dim);
@@ -815,6 +855,7 @@ extern "C" int fw_attention_decode_fused(const float* qkv, const float* q_norm_w
     FusedProjections fused;
     fused.qkv = qkv; fused.q_norm_weight = q_norm_weight; fused.k_norm_weight = k_norm_weight; fused.eps = eps;
     fused.cos_table = cos_table; fused.sin_table = sin_table; fused.rotary_dim = rotary_dim; fused.write_kv = write_kv;
+    fused.interleaved = interleaved;
     return decode_launch(nullptr, out, partial, max_splits, decode_work, tickets, k_pages, v_pages, block_table, table_stride, row_seg, row_pos,
-                         rows, num_heads, num_kv_heads, head_dim, v_dim, scale, window, fused, stream);
+                         rows, num_heads, num_kv_heads, head_dim, v_dim, scale, window, chunk, softcap, fused, stream);
 }

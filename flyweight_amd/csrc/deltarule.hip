@@ -36,7 +36,7 @@ __global__ __launch_bounds__(64) void delta_prepare_kernel(
     const TI* __restrict__ proj, int proj_stride, int beta_col, const TI* __restrict__ a, int a_stride, const float* __restrict__ taps,
     float* __restrict__ conv_state, const float* __restrict__ A_log, const float* __restrict__ dt_bias,
     const int32_t* __restrict__ row_seg, const int32_t* __restrict__ seg_row0, const int32_t* __restrict__ seg_slot,
-    float* __restrict__ records, int heads, int kv_heads, int dim, int vdim, int taps_count) {
+    float* __restrict__ records, int heads, int kv_heads, int dim, int vdim, int taps_count, int decay_per_head) {
     const int row = blockIdx.x, vec = blockIdx.y, lane = threadIdx.x;
     const int conv_channels = 2 * kv_heads * dim + heads * vdim;
     const int d4 = (dim + 3) & ~3, v4 = (vdim + 3) & ~3;
@@ -47,7 +47,7 @@ __global__ __launch_bounds__(64) void delta_prepare_kernel(
         const float rate = expf(A_log[h]);
         float* dest = of_row + (size_t)h * record + 2 * d4;
         for (int i = lane; i < d4; i += 64) {
-            const int at = h * dim + i;
+            const int at = decay_per_head ? h : h * dim + i;    // one decay for the head: every key channel gets it
             dest[i] = i < dim ? expf(-rate * fw_softplus(load_as_float(a, (size_t)row * a_stride + at) + dt_bias[at])) : 0.0f;
         }
         if (lane < 4) dest[d4 + lane] = lane == 0 ? fw_sigmoid(load_as_float(proj, (size_t)row * proj_stride + beta_col + h)) : 0.0f;
@@ -128,7 +128,8 @@ __global__ void conv_state_kernel(const TI* __restrict__ proj, int proj_stride, 
 extern "C" int fw_delta_prepare(const void* proj, int dtype, int proj_stride, int beta_col, const void* a, int a_stride, const float* taps,
                                 float* conv_state, const float* A_log, const float* dt_bias, const int32_t* row_seg,
                                 const int32_t* seg_row0, const int32_t* seg_slot, float* records, int rows, int segments,
-                                int heads, int kv_heads, int dim, int vdim, int taps_count, int slots, void* stream) {
+                                int heads, int kv_heads, int dim, int vdim, int taps_count, int slots, int decay_per_head,
+                                void* stream) {
     FW_REQUIRE(rows >= 0 && segments >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0,
                "delta_prepare: heads %d must be a positive multiple of kv heads %d", heads, kv_heads);
     FW_REQUIRE(dim > 0 && dim <= 256 && vdim > 0 && vdim <= 256, "delta_prepare: dim %d and vdim %d must lie in 1..256", dim, vdim);
@@ -137,7 +138,7 @@ extern "C" int fw_delta_prepare(const void* proj, int dtype, int proj_stride, in
     const int channels = 2 * kv_heads * dim + heads * vdim;
     FW_REQUIRE(proj_stride >= channels && beta_col >= 0 && beta_col + heads <= proj_stride,
                "delta_prepare: the projections' rows (%d wide) do not hold %d channels and %d strengths at %d", proj_stride, channels, heads, beta_col);
-    FW_REQUIRE(a_stride >= heads * dim, "delta_prepare: the decays' arguments (%d wide) do not hold %d x %d", a_stride, heads, dim);
+    FW_REQUIRE(a_stride >= (decay_per_head ? heads : heads * dim), "delta_prepare: the decays' arguments (%d wide) do not hold %d x %d", a_stride, heads, decay_per_head ? 1 : dim);
     FW_REQUIRE(rows <= 1 << 20 && segments <= 65535 && 2 * kv_heads + 2 * heads <= 65535, "delta_prepare: too many rows, segments or heads");
     if (rows == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
@@ -147,7 +148,7 @@ extern "C" int fw_delta_prepare(const void* proj, int dtype, int proj_stride, in
 #define FW_PREPARE_LAUNCH(TI, SINGLE)                                                                                         \
     delta_prepare_kernel<TI, SINGLE><<<grid, 64, 0, s>>>((const TI*)proj, proj_stride, beta_col, (const TI*)a, a_stride, taps, \
                                                          conv_state, A_log, dt_bias, row_seg, seg_row0, seg_slot, records,     \
-                                                         heads, kv_heads, dim, vdim, taps_count)
+                                                         heads, kv_heads, dim, vdim, taps_count, decay_per_head)
     if (dtype == FW_F32) {
         if (single) FW_PREPARE_LAUNCH(float, true);
         else FW_PREPARE_LAUNCH(float, false);
@@ -357,7 +358,7 @@ extern "C" int fw_gated_delta_rule(const float* records, float* state, float* ou
 template <typename TG, typename T>
 __global__ __launch_bounds__(64) void gated_head_norm_kernel(const float* __restrict__ o, const TG* __restrict__ gate, int gate_stride,
                                                             const float* __restrict__ weight, T* __restrict__ out,
-                                                            int heads, int vdim, float eps) {
+                                                            int heads, int vdim, float eps, int gate_silu) {
     const int row = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
     const float* source = o + ((size_t)row * heads + head) * vdim;
     float sum = 0.0f;
@@ -365,20 +366,21 @@ __global__ __launch_bounds__(64) void gated_head_norm_kernel(const float* __rest
     sum = wave_sum(sum);
     const float inv = 1.0f / sqrtf(sum / (float)vdim + eps);
     for (int j = lane; j < vdim; j += 64) {
-        const float g = fw_sigmoid(load_as_float(gate, (size_t)row * gate_stride + head * vdim + j));
+        const float z = load_as_float(gate, (size_t)row * gate_stride + head * vdim + j);
+        const float g = gate_silu ? z * fw_sigmoid(z) : fw_sigmoid(z);
         store_from_float(out, ((size_t)row * heads + head) * vdim + j, source[j] * inv * weight[j] * g);
     }
 }
 
 extern "C" int fw_gated_head_norm(const float* o, const void* gate, int gate_dtype, int gate_stride, const float* weight,
-                                  void* out, int out_dtype, int rows, int heads, int vdim, float eps, void* stream) {
+                                  void* out, int out_dtype, int rows, int heads, int vdim, float eps, int gate_silu, void* stream) {
     FW_REQUIRE(rows >= 0 && heads > 0 && heads <= 65535 && vdim > 0, "gated_head_norm: bad sizes rows=%d heads=%d vdim=%d", rows, heads, vdim);
     FW_REQUIRE(gate_stride >= heads * vdim, "gated_head_norm: the gates' rows (%d wide) do not hold %d x %d", gate_stride, heads, vdim);
     if (rows == 0) return 0;
     dim3 grid(rows, heads);
     hipStream_t s = (hipStream_t)stream;
 #define FW_GHN_LAUNCH(TG, T) \
-    gated_head_norm_kernel<TG, T><<<grid, 64, 0, s>>>(o, (const TG*)gate, gate_stride, weight, (T*)out, heads, vdim, eps)
+    gated_head_norm_kernel<TG, T><<<grid, 64, 0, s>>>(o, (const TG*)gate, gate_stride, weight, (T*)out, heads, vdim, eps, gate_silu)
     if (gate_dtype == FW_F32 && out_dtype == FW_F32) FW_GHN_LAUNCH(float, float);
     else if (gate_dtype == FW_F32 && out_dtype == FW_BF16) FW_GHN_LAUNCH(float, bf16_t);
     else if (gate_dtype == FW_BF16 && out_dtype == FW_BF16) FW_GHN_LAUNCH(bf16_t, bf16_t);

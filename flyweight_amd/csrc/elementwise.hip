@@ -16,7 +16,7 @@ void fw_set_error(const char* format, ...) {
     va_end(args);
 }
 extern "C" const char* fw_last_error(void) { return fw_error_text; }
-extern "C" int fw_abi_version(void) { return 12; }
+extern "C" int fw_abi_version(void) { return 13; }
 
 // ---- embedding -------------------------------------------------------------------------
 // The reference gathers one row per token and widens it to float32
@@ -378,5 +378,112 @@ extern "C" int fw_fill_zero(void* ptr, long long bytes, void* stream) {
     if (blocks > 2048) blocks = 2048;
     fill_zero_kernel<<<blocks, 256, 0, (hipStream_t)stream>>>((uint32_t*)ptr, words);
     FW_LAUNCH_CHECK("fill_zero");
+    return 0;
+}
+
+// ---- layer norm with a weight and no bias -----------------------------------------------------------
+// out[r] = (x[src] - mean) / sqrt(mean((x[src] - mean)^2) + eps) * w, src = row_index ? row_index[r] : r.
+// The mean first, then the mean of the squared deviations from it (not E[x^2] - mean^2, which loses
+// digits where the mean is large beside the spread). A row of up to 4,096 values stays in registers.
+template <typename T>
+__global__ __launch_bounds__(256) void layernorm_rows_kernel(const float* __restrict__ x, const float* __restrict__ weight,
+                                                             T* __restrict__ out, const int32_t* __restrict__ row_index,
+                                                             int hidden, float eps) {
+    __shared__ float scratch[16];
+    const int row = blockIdx.x;
+    const float* source = x + (size_t)(row_index ? row_index[row] : row) * hidden;
+    const bool held_all = hidden <= 256 * 16;
+    float held[16], scale[16];
+    float sum = 0.0f;
+    if (held_all) {
+#pragma unroll
+        for (int u = 0; u < 16; ++u) {
+            const int i = threadIdx.x + 256 * u;
+            held[u] = i < hidden ? source[i] : 0.0f;
+            scale[u] = i < hidden ? weight[i] : 0.0f;
+            sum += held[u];
+        }
+    } else {
+        for (int i = threadIdx.x; i < hidden; i += 256) sum += source[i];
+    }
+    const float mean = block_sum(sum, scratch) / (float)hidden;
+    float squares = 0.0f;
+    if (held_all) {
+#pragma unroll
+        for (int u = 0; u < 16; ++u) {
+            const float d = threadIdx.x + 256 * u < hidden ? held[u] - mean : 0.0f;
+            squares = fmaf(d, d, squares);
+        }
+    } else {
+        for (int i = threadIdx.x; i < hidden; i += 256) {
+            const float d = source[i] - mean;
+            squares = fmaf(d, d, squares);
+        }
+    }
+    const float inv = 1.0f / sqrtf(block_sum(squares, scratch) / (float)hidden + eps);
+    if (held_all) {
+#pragma unroll
+        for (int u = 0; u < 16; ++u) {
+            const int i = threadIdx.x + 256 * u;
+            if (i < hidden) store_from_float(out, (size_t)row * hidden + i, (held[u] - mean) * inv * scale[u]);
+        }
+    } else {
+        for (int i = threadIdx.x; i < hidden; i += 256)
+            store_from_float(out, (size_t)row * hidden + i, (source[i] - mean) * inv * weight[i]);
+    }
+}
+
+extern "C" int fw_layernorm_rows(const float* x, const float* weight, void* out, int out_dtype, const int32_t* row_index,
+                                 int rows, int hidden, float eps, void* stream) {
+    FW_REQUIRE(rows >= 0 && hidden > 0, "layernorm_rows: bad sizes rows=%d hidden=%d", rows, hidden);
+    FW_REQUIRE(eps > 0.0f, "layernorm_rows: eps must be positive");
+    if (rows == 0) return 0;
+    if (out_dtype == FW_F32)
+        layernorm_rows_kernel<float><<<rows, 256, 0, (hipStream_t)stream>>>(x, weight, (float*)out, row_index, hidden, eps);
+    else if (out_dtype == FW_BF16)
+        layernorm_rows_kernel<bf16_t><<<rows, 256, 0, (hipStream_t)stream>>>(x, weight, (bf16_t*)out, row_index, hidden, eps);
+    else
+        FW_REQUIRE(false, "layernorm_rows: unknown out dtype %d", out_dtype);
+    FW_LAUNCH_CHECK("layernorm_rows");
+    return 0;
+}
+
+// ---- a gate on a row of a second token table ----------------------------------------------------------
+// out[r][j] = gelu_tanh(z[r][j]) * table[ids[r]][col0 + j], j < width, where
+// gelu_tanh(z) = 0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3))). z float32 [rows][z_stride].
+template <typename TT, typename TO>
+__global__ void gelu_gate_rows_kernel(const float* __restrict__ z, int z_stride, const TT* __restrict__ table, int table_width,
+                                      int col0, const int32_t* __restrict__ ids, TO* __restrict__ out, int width) {
+    const int row = blockIdx.y;
+    const TT* entry = table + (size_t)ids[row] * table_width + col0;
+    for (int j = blockIdx.x * blockDim.x + threadIdx.x; j < width; j += gridDim.x * blockDim.x) {
+        const float v = z[(size_t)row * z_stride + j];
+        const float gelu = 0.5f * v * (1.0f + tanhf(0.7978845608028654f * (v + 0.044715f * v * v * v)));
+        store_from_float(out, (size_t)row * width + j, gelu * load_as_float(entry, j));
+    }
+}
+
+extern "C" int fw_gelu_gate_rows(const float* z, int z_stride, const void* table, int table_dtype, int table_rows, int table_width,
+                                 int col0, const int32_t* ids, void* out, int out_dtype, int rows, int width, void* stream) {
+    FW_REQUIRE(rows >= 0 && width > 0 && z_stride >= width, "gelu_gate_rows: bad sizes rows=%d width=%d stride=%d", rows, width, z_stride);
+    FW_REQUIRE(table_rows > 0 && col0 >= 0 && col0 + width <= table_width, "gelu_gate_rows: columns %d..%d lie outside the table's %d", col0, col0 + width, table_width);
+    if (rows == 0) return 0;
+    int across = (width + 255) / 256;
+    if (across > 64) across = 64;
+    hipStream_t s = (hipStream_t)stream;
+    for (int row0 = 0; row0 < rows; row0 += 65535) {
+        const int now = rows - row0 < 65535 ? rows - row0 : 65535;
+        dim3 grid(across, now);
+#define FW_GATE_LAUNCH(TT, TO)                                                                                               \
+    gelu_gate_rows_kernel<TT, TO><<<grid, 256, 0, s>>>(z + (size_t)row0 * z_stride, z_stride, (const TT*)table, table_width, \
+                                                       col0, ids + row0, (TO*)out + (size_t)row0 * width, width)
+        if (table_dtype == FW_F32 && out_dtype == FW_F32) FW_GATE_LAUNCH(float, float);
+        else if (table_dtype == FW_BF16 && out_dtype == FW_BF16) FW_GATE_LAUNCH(bf16_t, bf16_t);
+        else if (table_dtype == FW_BF16 && out_dtype == FW_F32) FW_GATE_LAUNCH(bf16_t, float);
+        else if (table_dtype == FW_F32 && out_dtype == FW_BF16) FW_GATE_LAUNCH(float, bf16_t);
+        else FW_REQUIRE(false, "gelu_gate_rows: unsupported dtypes table=%d out=%d", table_dtype, out_dtype);
+#undef FW_GATE_LAUNCH
+    }
+    FW_LAUNCH_CHECK("gelu_gate_rows");
     return 0;
 }

@@ -169,6 +169,18 @@ __device__ __forceinline__ float fw_gated_unit(float g, float u, float limit, fl
     return g * (z >= 0.0f ? 1.0f / (1.0f + e) : e / (1.0f + e)) * (u + shift);
 }
 
+// The first key that a row at position `pos` may see: with a window the last `window` keys (itself
+// among them), with a chunk only the keys of its own chunk (chunks counted from position 0 of the
+// sequence); 0 switches either off. Never falls as the position rises.
+__host__ __device__ __forceinline__ int fw_first_visible(int pos, int window, int chunk) {
+    int first = window > 0 && pos - window + 1 > 0 ? pos - window + 1 : 0;
+    if (chunk > 0) {
+        const int start = pos - pos % chunk;
+        first = start > first ? start : first;
+    }
+    return first;
+}
+
 static inline int fw_ceil_div(long long a, long long b) { return (int)((a + b - 1) / b); }
 
 // Eight bfloat16 of a weight matrix that a decode step reads once: with `streamed` the load says

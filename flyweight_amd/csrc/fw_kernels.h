@@ -121,8 +121,9 @@ int fw_shortconv(const void* bcx, int in_dtype, void* out, int out_dtype, const 
                  const int32_t* seg_slot, int rows, int segments, int hidden, int kernel_size,
                  int slots, void* stream);
 
-// Per-head RMS norm of q and k (weights may be null: no norm), half-split rotation of the
-// first rotary_dim channels by the row's angle, q out, k and v appended to the pages of
+// Per-head RMS norm of q and k (weights may be null: no norm), rotation of the
+// first rotary_dim channels by the row's angle (interleaved 0: channel i turns with channel i + rotary_dim / 2;
+// 1: channel 2i with channel 2i + 1; the tables are the same), q out, k and v appended to the pages of
 // the row's segment. qkv [rows][(nh + nkv) hd + nkv vd]: values may have a size vd of their own.
 // k_pages [pages][nkv][P][hd]; v_pages [pages][nkv][vd][P]. block_table [segments][table_stride].
 int fw_qk_norm_rope_kv_write(const void* qkv, int in_dtype, void* q_out, int dtype, const float* q_norm_weight,
@@ -130,15 +131,16 @@ int fw_qk_norm_rope_kv_write(const void* qkv, int in_dtype, void* q_out, int dty
                              const float* sin_table, int rotary_dim, void* k_pages, void* v_pages,
                              const int32_t* block_table, int table_stride, const int32_t* row_seg,
                              const int32_t* row_pos, int rows, int num_heads, int num_kv_heads,
-                             int head_dim, int v_dim, int page_size, int num_pages, int write_kv, void* stream);
+                             int head_dim, int v_dim, int page_size, int num_pages, int write_kv, int interleaved, void* stream);
 
-// Causal attention of every row over the cached keys 0..row_pos[r] (or the last `window`
-// of them) of its segment. out [rows][nh*vd].
+// Causal attention of every row over the cached keys 0..row_pos[r] of its segment, or the last `window`
+// of them, or with `chunk` > 0 those of its own chunk of that many positions (counted from position 0
+// of the sequence); softcap c > 0: score <- c * tanh(score / c) after the scale. out [rows][nh*vd].
 int fw_attention_generic(const void* q, void* out, int dtype, const void* k_pages,
                          const void* v_pages, const int32_t* block_table, int table_stride,
                          const int32_t* row_seg, const int32_t* row_pos, int rows, int num_heads,
-                         int num_kv_heads, int head_dim, int v_dim, float scale, int window, int page_size,
-                         int num_pages, void* stream);
+                         int num_kv_heads, int head_dim, int v_dim, float scale, int window, int chunk, float softcap,
+                         int page_size, int num_pages, void* stream);
 
 // The same attention on the matrix cores, bfloat16 only, head_dim and v_dim (the size of a value and of a
 // head's output: out [rows][nh * v_dim]) multiples of 16 up to 256.
@@ -151,7 +153,7 @@ int fw_attention_prefill(const void* q, void* out, const void* k_pages, const vo
                          const int32_t* block_table, int table_stride, const int32_t* tile_seg,
                          const int32_t* tile_row0, int tiles, const int32_t* seg_row0, const int32_t* row_pos,
                          int rows, int num_heads, int num_kv_heads, int head_dim, int v_dim, float scale, int window,
-                         int page_size, int num_pages, int heads_together, void* stream);
+                         int chunk, float softcap, int page_size, int num_pages, int heads_together, void* stream);
 // Decode (one row per request): the keys are split between workgroups in runs of 4 pages and
 // merged in order by the workgroup that finishes last. partial: float32 workspace
 // [rows][heads][max_splits][v_dim + 4]; max_context: an upper bound on position + 1 of every
@@ -162,7 +164,8 @@ int fw_attention_prefill(const void* q, void* out, const void* k_pages, const vo
 int fw_attention_decode(const void* q, void* out, float* partial, int max_splits, int max_context,
                         const int32_t* decode_work, int* tickets, int tickets_len, const void* k_pages, const void* v_pages, const int32_t* block_table, int table_stride,
                         const int32_t* row_seg, const int32_t* row_pos, int rows, int num_heads, int num_kv_heads,
-                        int head_dim, int v_dim, float scale, int window, int page_size, int num_pages, void* stream);
+                        int head_dim, int v_dim, float scale, int window, int chunk, float softcap, int page_size, int num_pages,
+                        void* stream);
 
 // The same with the work of fw_qk_norm_rope_kv_write in front of it, in one kernel: qkv float32
 // [rows][(heads + kv_heads) * head_dim + kv_heads * v_dim] are the step's raw projections; every workgroup norms and
@@ -174,7 +177,8 @@ int fw_attention_decode_fused(const float* qkv, const float* q_norm_weight, cons
                               int tickets_len, void* k_pages,
                               void* v_pages, const int32_t* block_table, int table_stride, const int32_t* row_seg,
                               const int32_t* row_pos, int rows, int num_heads, int num_kv_heads, int head_dim, int v_dim,
-                              float scale, int window, int page_size, int num_pages, void* stream);
+                              float scale, int window, int chunk, float softcap, int interleaved, int page_size, int num_pages,
+                              void* stream);
 
 // ids[r] = argmax(logits[r]) with ties to the lowest id, also written to also[r] if that is not null;
 // advance[r] += 1 if that is not null; workspace: rows * 64 64-bit words
@@ -201,6 +205,16 @@ int fw_argmax_rows_static_max_rows(void);
 int fw_sample_rows(const float* logits, const float* settings, unsigned long long* states, int32_t* ids, int32_t* also,
                    int32_t* advance, int rows, int vocab, void* stream);
 
+// Layer norm with a weight and no bias: out[r] = (x[src] - mean) / sqrt(mean((x[src] - mean)^2) + eps) * w,
+// src = row_index ? row_index[r] : r.
+int fw_layernorm_rows(const float* x, const float* weight, void* out, int out_dtype, const int32_t* row_index,
+                      int rows, int hidden, float eps, void* stream);
+
+// out[r][j] = gelu_tanh(z[r][j]) * table[ids[r]][col0 + j] for j < width; z float32 [rows][z_stride],
+// table [table_rows][table_width] (a second token table of which a layer reads its own columns).
+int fw_gelu_gate_rows(const float* z, int z_stride, const void* table, int table_dtype, int table_rows, int table_width,
+                      int col0, const int32_t* ids, void* out, int out_dtype, int rows, int width, void* stream);
+
 int fw_fill_zero(void* ptr, long long bytes, void* stream);
 // `pieces` runs of `bytes` each, `stride_bytes` apart, cleared in one launch
 int fw_fill_zero_pieces(void* ptr, int pieces, long long bytes, long long stride_bytes, void* stream);
@@ -216,21 +230,23 @@ int fw_fill_zero_pieces(void* ptr, int pieces, long long bytes, long long stride
 // [channels][L], the last column the current token's; conv_state [slots][channels][L - 1], oldest
 // first, read and then moved on by the segment's rows. q, k, v are the silu of the convolutions, q and
 // k of unit length per head (sum of squares + 1e-6 under the root), q also times d^-1/2;
-// g = exp(-exp(A_log[h]) * softplus(a + dt_bias)).
+// g = exp(-exp(A_log[h]) * softplus(a + dt_bias)). decay_per_head: a holds one argument per head
+// (its first H columns) and dt_bias [H]; every key channel of the head then decays alike.
 int fw_delta_record_floats(int dim, int vdim);
 int fw_delta_prepare(const void* proj, int dtype, int proj_stride, int beta_col, const void* a, int a_stride, const float* taps,
                      float* conv_state, const float* A_log, const float* dt_bias, const int32_t* row_seg,
                      const int32_t* seg_row0, const int32_t* seg_slot, float* records, int rows, int segments,
-                     int heads, int kv_heads, int dim, int vdim, int taps_count, int slots, void* stream);
+                     int heads, int kv_heads, int dim, int vdim, int taps_count, int slots, int decay_per_head, void* stream);
 // Per segment and head, token by token: S <- diag(g) S; u = beta (v - S^T k); S <- S + k u^T;
 // o = S^T q. records [rows][H][fw_delta_record_floats]. state [slots][H][vd][d] (S transposed), read
 // at the segment's start and written at its end. out [rows][H vd].
 int fw_gated_delta_rule(const float* records, float* state, float* out, const int32_t* seg_row0,
                         const int32_t* seg_slot, int rows, int segments, int heads, int dim, int vdim,
                         int slots, void* stream);
-// out[r][h][j] = o[r][h][j] * rsqrt(mean_j o[r][h]^2 + eps) * weight[j] * sigmoid(gate[r][h vd + j])
+// out[r][h][j] = o[r][h][j] * rsqrt(mean_j o[r][h]^2 + eps) * weight[j] * act(gate[r][h vd + j]);
+// act is the sigmoid, or with gate_silu z * sigmoid(z)
 int fw_gated_head_norm(const float* o, const void* gate, int gate_dtype, int gate_stride, const float* weight,
-                       void* out, int out_dtype, int rows, int heads, int vdim, float eps, void* stream);
+                       void* out, int out_dtype, int rows, int heads, int vdim, float eps, int gate_silu, void* stream);
 
 // ---- sublayers whose output is normed ------------------------------------------------------------
 // x[r] += mult * rmsnorm(scale_a a[r] + scale_b b[r]) * w (b may be null; one_centered: 1 + w);
@@ -238,12 +254,32 @@ int fw_gated_head_norm(const float* o, const void* gate, int gate_dtype, int gat
 int fw_norm_scale_add(float* x, const float* a, const float* b, float scale_a, float scale_b, const float* weight,
                       int one_centered, float eps, float mult, void* rounded, int rounded_dtype, int rows,
                       int hidden, void* stream);
+// A sublayer between two norms: x[r] += norm(a[r]) * weight (RMS: a / sqrt(mean(a^2) + eps); centered: the
+// row's mean taken off first), and what reads x next, formed from the new row in the same pass:
+// next_kind 0 nothing, 1 x rounded to next_dtype, 2 the RMS norm of x times next_weight, 3 the same with
+// the mean taken off (next_eps under its root); next_out [rows][hidden] of next_dtype.
+int fw_norm_add_norm(float* x, const float* a, const float* weight, int centered, float eps, int next_kind,
+                     const float* next_weight, float next_eps, void* next_out, int next_dtype, int rows, int hidden,
+                     void* stream);
 // out (bfloat16) = x (float32), count elements
 int fw_round_rows(const float* x, void* out, long long count, void* stream);
 // gate_up [rows][2 I]: out[r][i] = g sigmoid(alpha g) (u + shift), g = min(gate, limit),
 // u = clamp(up, -limit, limit)
 int fw_clamped_glu(const void* gate_up, int in_dtype, void* out, int out_dtype, int rows, int intermediate,
                    float limit, float alpha, float shift, void* stream);
+
+// ---- attention over a cached latent ---------------------------------------------------------------
+// The latent of a step's rows: columns col0 .. col0 + rank - 1 of raw [rows][raw_stride] (float32), RMS-normed
+// (eps under the root) times weight [rank], stored at each row's position in both layouts of a cache
+// with one key/value head of `rank` channels: k_pages [pages][1][P][rank], v_pages [pages][1][rank][P].
+int fw_latent_norm_write(const float* raw, int raw_stride, int col0, const float* weight, float eps, void* k_pages,
+                         void* v_pages, int dtype, const int32_t* block_table, int table_stride, const int32_t* row_seg,
+                         const int32_t* row_pos, int rows, int rank, int page_size, int num_pages, void* stream);
+// A map per head: out[r][h N + n] = sum_k in[r][h K + k] * w[h][n][k], with a gate (may be null) times
+// sigmoid(gate[r][h N + n]). in [rows][in_stride], w [heads][N][K], gate float32 [rows][gate_stride],
+// out [rows][heads N].
+int fw_head_linear(const void* in, int in_dtype, int in_stride, const void* w, int w_dtype, const float* gate, int gate_stride,
+                   void* out, int out_dtype, int rows, int heads, int N, int K, void* stream);
 
 #ifdef __cplusplus
 }

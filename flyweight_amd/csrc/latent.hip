@@ -1,0 +1,141 @@
+// Attention over a cached latent: keys and values of every head are linear maps of one normed
+// vector c per token (k_h = U_h c, v_h = V_h c), so only c is cached and the maps move to the
+// query's side: score = q_h . (U_h c) = (U_h^T q_h) . c, and the head's output V_h (sum_j p_j c_j).
+// The attention kernels then see one shared key/value head of the latent's size. Here: the norm of
+// the latent with its store into the pages, and the per-head maps on the query's and the output's side.
+#include "fw_common.h"
+#include "fw_kernels.h"
+
+#define LATENT_PAGE 64
+
+// ---- the latent of a step's rows, normed and stored ---------------------------------------------------
+// raw [rows][raw_stride] float32 holds the latent before its norm in columns col0 .. col0 + rank - 1.
+// c = raw / sqrt(mean(raw^2) + eps) * weight goes to both layouts of the cache's one head:
+// k_pages [page][1][64][rank] (a token's channels together) and v_pages [page][1][rank][64].
+template <typename T>
+__global__ __launch_bounds__(256) void latent_norm_write_kernel(
+    const float* __restrict__ raw, int raw_stride, int col0, const float* __restrict__ weight, float eps,
+    T* __restrict__ k_pages, T* __restrict__ v_pages, const int32_t* __restrict__ block_table, int table_stride,
+    const int32_t* __restrict__ row_seg, const int32_t* __restrict__ row_pos, int rank) {
+    __shared__ float scratch[16];
+    const int row = blockIdx.x;
+    const float* source = raw + (size_t)row * raw_stride + col0;
+    const int pos = row_pos[row];
+    const int page = block_table[(size_t)row_seg[row] * table_stride + pos / LATENT_PAGE];
+    const int slot = pos % LATENT_PAGE;
+    float sum = 0.0f;
+    for (int j = threadIdx.x; j < rank; j += 256) sum = fmaf(source[j], source[j], sum);
+    const float inv = 1.0f / sqrtf(block_sum(sum, scratch) / (float)rank + eps);
+    T* key = k_pages + ((size_t)page * LATENT_PAGE + slot) * rank;
+    T* value = v_pages + (size_t)page * rank * LATENT_PAGE + slot;
+    for (int j = threadIdx.x; j < rank; j += 256) {
+        const float c = source[j] * inv * weight[j];
+        store_from_float(key, j, c);
+        store_from_float(value, (size_t)j * LATENT_PAGE, c);
+    }
+}
+
+extern "C" int fw_latent_norm_write(const float* raw, int raw_stride, int col0, const float* weight, float eps, void* k_pages,
+                                    void* v_pages, int dtype, const int32_t* block_table, int table_stride,
+                                    const int32_t* row_seg, const int32_t* row_pos, int rows, int rank, int page_size,
+                                    int num_pages, void* stream) {
+    FW_REQUIRE(rows >= 0 && rank > 0 && col0 >= 0 && col0 + rank <= raw_stride, "latent_norm_write: columns %d..%d of rows %d wide", col0,
+               col0 + rank, raw_stride);
+    FW_REQUIRE(eps > 0.0f, "latent_norm_write: eps must be positive");
+    FW_REQUIRE(page_size == LATENT_PAGE, "latent_norm_write: page size must be %d, got %d", LATENT_PAGE, page_size);
+    FW_REQUIRE(num_pages > 0 && table_stride > 0, "latent_norm_write: empty cache (pages=%d, table stride=%d)", num_pages, table_stride);
+    if (rows == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    if (dtype == FW_F32)
+        latent_norm_write_kernel<float><<<rows, 256, 0, s>>>(raw, raw_stride, col0, weight, eps, (float*)k_pages, (float*)v_pages,
+                                                             block_table, table_stride, row_seg, row_pos, rank);
+    else if (dtype == FW_BF16)
+        latent_norm_write_kernel<bf16_t><<<rows, 256, 0, s>>>(raw, raw_stride, col0, weight, eps, (bf16_t*)k_pages, (bf16_t*)v_pages,
+                                                              block_table, table_stride, row_seg, row_pos, rank);
+    else
+        FW_REQUIRE(false, "latent_norm_write: unknown dtype %d", dtype);
+    FW_LAUNCH_CHECK("latent_norm_write");
+    return 0;
+}
+
+// ---- a map per head ------------------------------------------------------------------------------------
+// out[r][h N + n] = sum_k in[r][h K + k] * w[h][n][k], then with a gate (float32) times sigmoid(gate[r][h N + n]).
+// in [rows][in_stride], w [heads][N][K], out [rows][heads N]. Float32 sums, each output summed over k
+// in order by one thread: a function of the row alone.
+#define HL_TILE 64          // rows and columns of a workgroup's tile
+#define HL_K 16             // k values staged at a time
+template <typename TI, typename TW, typename TO>
+__global__ __launch_bounds__(256) void head_linear_kernel(const TI* __restrict__ in, int in_stride, const TW* __restrict__ w,
+                                                         const float* __restrict__ gate, int gate_stride, TO* __restrict__ out,
+                                                         int rows, int heads, int N, int K) {
+    __shared__ float a_tile[HL_K][HL_TILE + 1], w_tile[HL_K][HL_TILE + 1];
+    const int head = blockIdx.z;
+    const int row0 = blockIdx.x * HL_TILE, col0 = blockIdx.y * HL_TILE;
+    const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+    const TW* w_head = w + (size_t)head * N * K;
+    float acc[4][4] = {};
+    for (int k0 = 0; k0 < K; k0 += HL_K) {
+        // 64 x 16 of each operand: four values a thread
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int item = threadIdx.x + 256 * u;
+            const int line = item / HL_K, k = item % HL_K;
+            const bool k_in = k0 + k < K;
+            a_tile[k][line] = (k_in && row0 + line < rows) ? load_as_float(in, (size_t)(row0 + line) * in_stride + (size_t)head * K + k0 + k) : 0.0f;
+            w_tile[k][line] = (k_in && col0 + line < N) ? load_as_float(w_head, (size_t)(col0 + line) * K + k0 + k) : 0.0f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < HL_K; ++k) {
+            float av[4], wv[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                av[i] = a_tile[k][ty + 16 * i];
+                wv[i] = w_tile[k][tx + 16 * i];
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(av[i], wv[j], acc[i][j]);
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int row = row0 + ty + 16 * i;
+        if (row >= rows) continue;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int col = col0 + tx + 16 * j;
+            if (col >= N) continue;
+            float value = acc[i][j];
+            if (gate) {
+                const float z = gate[(size_t)row * gate_stride + (size_t)head * N + col];
+                value *= 1.0f / (1.0f + expf(-z));
+            }
+            store_from_float(out, (size_t)row * heads * N + (size_t)head * N + col, value);
+        }
+    }
+}
+
+extern "C" int fw_head_linear(const void* in, int in_dtype, int in_stride, const void* w, int w_dtype, const float* gate,
+                              int gate_stride, void* out, int out_dtype, int rows, int heads, int N, int K, void* stream) {
+    FW_REQUIRE(rows >= 0 && heads > 0 && heads <= 65535 && N > 0 && K > 0, "head_linear: bad sizes rows=%d heads=%d N=%d K=%d", rows, heads, N, K);
+    FW_REQUIRE(in_stride >= heads * K, "head_linear: rows %d wide do not hold %d x %d", in_stride, heads, K);
+    FW_REQUIRE(gate == nullptr || gate_stride >= heads * N, "head_linear: the gates' rows (%d wide) do not hold %d x %d", gate_stride, heads, N);
+    if (rows == 0) return 0;
+    dim3 grid((rows + HL_TILE - 1) / HL_TILE, (N + HL_TILE - 1) / HL_TILE, heads);
+    FW_REQUIRE(grid.y <= 65535, "head_linear: too many columns (%d)", N);
+    hipStream_t s = (hipStream_t)stream;
+#define FW_HL_LAUNCH(TI, TW, TO)                                                                                          \
+    head_linear_kernel<TI, TW, TO><<<grid, 256, 0, s>>>((const TI*)in, in_stride, (const TW*)w, gate, gate_stride, \
+                                                        (TO*)out, rows, heads, N, K)
+    if (in_dtype == FW_F32 && w_dtype == FW_F32 && out_dtype == FW_F32) FW_HL_LAUNCH(float, float, float);
+    else if (in_dtype == FW_BF16 && w_dtype == FW_BF16 && out_dtype == FW_BF16) FW_HL_LAUNCH(bf16_t, bf16_t, bf16_t);
+    else if (in_dtype == FW_BF16 && w_dtype == FW_BF16 && out_dtype == FW_F32) FW_HL_LAUNCH(bf16_t, bf16_t, float);
+    else if (in_dtype == FW_F32 && w_dtype == FW_BF16 && out_dtype == FW_BF16) FW_HL_LAUNCH(float, bf16_t, bf16_t);
+    else FW_REQUIRE(false, "head_linear: unsupported dtypes in=%d w=%d out=%d", in_dtype, w_dtype, out_dtype);
+#undef FW_HL_LAUNCH
+    FW_LAUNCH_CHECK("head_linear");
+    return 0;
+}

@@ -141,3 +141,137 @@ extern "C" int fw_clamped_glu(const void* gate_up, int in_dtype, void* out, int 
     FW_LAUNCH_CHECK("clamped_glu");
     return 0;
 }
+
+// ---- a sublayer between two norms ---------------------------------------------------------------------
+// What joins a sublayer whose output passes a norm of its own to the residual stream, and hands the
+// stream to the next reader, in one pass over the row:
+//     x <- x + norm_a(a) * w            (norm_a: RMS, or with `centered` the mean taken off first)
+//     next_out = next(x)                (next_kind 0: nothing; 1: x rounded to next_dtype; 2: RMS norm
+//                                        of x times next_weight; 3: the same with the mean taken off)
+// A norm here is v / sqrt(mean(v^2) + eps), v the values or their deviations from the row's mean. One
+// workgroup per row; a row of up to 256 * JOIN_HELD values stays in registers between the passes, a
+// wider one is read again. Every sum is a function of the row alone.
+#define JOIN_HELD 16
+template <typename T, bool HELD>
+__global__ __launch_bounds__(256) void norm_add_norm_kernel(
+    float* __restrict__ x, const float* __restrict__ a, const float* __restrict__ weight, int centered, float eps,
+    int next_kind, const float* __restrict__ next_weight, float next_eps, T* __restrict__ next_out, int hidden) {
+    __shared__ float scratch[16];
+    const size_t row0 = (size_t)blockIdx.x * hidden;
+    constexpr int N = HELD ? JOIN_HELD : 1;
+    float held[N], was[N], scale[N];
+    const float count = (float)hidden;
+    float sum = 0.0f;
+    if (HELD) {
+#pragma unroll
+        for (int u = 0; u < N; ++u) {
+            const int i = threadIdx.x + 256 * u;
+            const bool in = i < hidden;
+            held[u] = in ? a[row0 + i] : 0.0f;
+            was[u] = in ? x[row0 + i] : 0.0f;
+            scale[u] = in ? weight[i] : 0.0f;
+            sum += held[u];
+        }
+    } else {
+        for (int i = threadIdx.x; i < hidden; i += 256) sum += a[row0 + i];
+    }
+    const float mean = centered ? block_sum(sum, scratch) / count : 0.0f;
+    float squares = 0.0f;
+    if (HELD) {
+#pragma unroll
+        for (int u = 0; u < N; ++u) {
+            const float d = threadIdx.x + 256 * u < hidden ? held[u] - mean : 0.0f;
+            squares = fmaf(d, d, squares);
+        }
+    } else {
+        for (int i = threadIdx.x; i < hidden; i += 256) {
+            const float d = a[row0 + i] - mean;
+            squares = fmaf(d, d, squares);
+        }
+    }
+    const float inv = 1.0f / sqrtf(block_sum(squares, scratch) / count + eps);
+    float new_sum = 0.0f;
+    if (HELD) {
+#pragma unroll
+        for (int u = 0; u < N; ++u) {
+            const int i = threadIdx.x + 256 * u;
+            if (i < hidden) {
+                was[u] += (held[u] - mean) * inv * scale[u];
+                x[row0 + i] = was[u];
+                new_sum += was[u];
+            }
+        }
+    } else {
+        for (int i = threadIdx.x; i < hidden; i += 256) {
+            const float updated = x[row0 + i] + (a[row0 + i] - mean) * inv * weight[i];
+            x[row0 + i] = updated;          // read again below by the thread that wrote it
+            new_sum += updated;
+        }
+    }
+    if (next_kind == 0) return;
+    if (next_kind == 1) {
+        if (HELD) {
+#pragma unroll
+            for (int u = 0; u < N; ++u) {
+                const int i = threadIdx.x + 256 * u;
+                if (i < hidden) store_from_float(next_out, row0 + i, was[u]);
+            }
+        } else {
+            for (int i = threadIdx.x; i < hidden; i += 256) store_from_float(next_out, row0 + i, x[row0 + i]);
+        }
+        return;
+    }
+    const float next_mean = next_kind == 3 ? block_sum(new_sum, scratch) / count : 0.0f;
+    float next_squares = 0.0f;
+    if (HELD) {
+#pragma unroll
+        for (int u = 0; u < N; ++u) {
+            const float d = threadIdx.x + 256 * u < hidden ? was[u] - next_mean : 0.0f;
+            next_squares = fmaf(d, d, next_squares);
+        }
+    } else {
+        for (int i = threadIdx.x; i < hidden; i += 256) {
+            const float d = x[row0 + i] - next_mean;
+            next_squares = fmaf(d, d, next_squares);
+        }
+    }
+    const float next_inv = 1.0f / sqrtf(block_sum(next_squares, scratch) / count + next_eps);
+    if (HELD) {
+#pragma unroll
+        for (int u = 0; u < N; ++u) {
+            const int i = threadIdx.x + 256 * u;
+            if (i < hidden) store_from_float(next_out, row0 + i, (was[u] - next_mean) * next_inv * next_weight[i]);
+        }
+    } else {
+        for (int i = threadIdx.x; i < hidden; i += 256)
+            store_from_float(next_out, row0 + i, (x[row0 + i] - next_mean) * next_inv * next_weight[i]);
+    }
+}
+
+extern "C" int fw_norm_add_norm(float* x, const float* a, const float* weight, int centered, float eps, int next_kind,
+                                const float* next_weight, float next_eps, void* next_out, int next_dtype, int rows,
+                                int hidden, void* stream) {
+    FW_REQUIRE(rows >= 0 && hidden > 0, "norm_add_norm: bad sizes rows=%d hidden=%d", rows, hidden);
+    FW_REQUIRE(eps > 0.0f, "norm_add_norm: eps must be positive");
+    FW_REQUIRE(x && a && weight, "norm_add_norm: x, a and the weight are needed");
+    FW_REQUIRE(next_kind >= 0 && next_kind <= 3, "norm_add_norm: unknown kind %d of what follows", next_kind);
+    FW_REQUIRE(next_kind == 0 || next_out, "norm_add_norm: what follows has nowhere to go");
+    FW_REQUIRE(next_kind < 2 || (next_weight && next_eps > 0.0f), "norm_add_norm: the norm that follows needs a weight and a positive eps");
+    FW_REQUIRE(next_kind == 0 || next_dtype == FW_F32 || next_dtype == FW_BF16, "norm_add_norm: unknown dtype %d", next_dtype);
+    if (rows == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    const bool held = hidden <= 256 * JOIN_HELD;
+#define FW_JOIN_LAUNCH(T, HELD)                                                                                             \
+    norm_add_norm_kernel<T, HELD><<<rows, 256, 0, s>>>(x, a, weight, centered, eps, next_kind, next_weight, next_eps, \
+                                                       (T*)next_out, hidden)
+    if (next_kind == 0 || next_dtype == FW_F32) {
+        if (held) FW_JOIN_LAUNCH(float, true);
+        else FW_JOIN_LAUNCH(float, false);
+    } else {
+        if (held) FW_JOIN_LAUNCH(bf16_t, true);
+        else FW_JOIN_LAUNCH(bf16_t, false);
+    }
+#undef FW_JOIN_LAUNCH
+    FW_LAUNCH_CHECK("norm_add_norm");
+    return 0;
+}

@@ -14,7 +14,7 @@ import sys
 from typing import IO, List, Optional
 
 PAGE_SIZE = 64
-MAX_LIVE_SLOTS = 64     # state slots are memory per request: bounded even when the pool is large
+LIVE_REQUESTS = 4       # state slots are memory per request: as many as requests are live at once, and used again
 
 
 def build_parser() -> argparse.ArgumentParser:
@@ -28,26 +28,27 @@ def build_parser() -> argparse.ArgumentParser:
     parser.add_argument("--out", required=True, metavar="DIR", help="where the logits files go")
     parser.add_argument("--max-tokens", required=True, type=int, metavar="N",
                         help="the most tokens live requests hold at any time, each request rounded up to a multiple "
-                             f"of {PAGE_SIZE}; the cache pool is made for this many. As many requests may be live "
-                             f"as the pool has pages (a request holds at least one), at most {MAX_LIVE_SLOTS}")
+                             f"of {PAGE_SIZE}; the cache pool is made for this many")
+    parser.add_argument("--max-requests", type=int, default=LIVE_REQUESTS, metavar="N",
+                        help=f"the most requests that are live at any time: the engine has this many state slots (default {LIVE_REQUESTS})")
     parser.add_argument("--device", default="cuda:0", help=argparse.SUPPRESS)
     return parser
 
 
 def replay(model_dir: str, dtype: str, out_dir: str, max_tokens: int, lines: IO[str], done: IO[str],
-           device: str = "cuda:0") -> int:
+           device: str = "cuda:0", max_requests: int = LIVE_REQUESTS) -> int:
     import numpy as np
     import torch
 
     from .model import load_model
     from .step import StepEntry, Stepper
 
-    if max_tokens <= 0:
-        raise ValueError("--max-tokens must be positive")
+    if max_tokens <= 0 or max_requests <= 0:
+        raise ValueError("--max-tokens and --max-requests must be positive")
     os.makedirs(out_dir, exist_ok=True)
     _, model = load_model(model_dir, dtype=dtype, device=device)
     num_pages = (max_tokens + PAGE_SIZE - 1) // PAGE_SIZE
-    stepper = Stepper(model, num_pages=num_pages, max_requests=min(num_pages, MAX_LIVE_SLOTS), page_size=PAGE_SIZE,
+    stepper = Stepper(model, num_pages=num_pages, max_requests=max_requests, page_size=PAGE_SIZE,
                       context_limit=min(model.spec.max_positions, num_pages * PAGE_SIZE))
     for number, line in enumerate(lines):
         line = line.strip()
@@ -80,7 +81,8 @@ def replay(model_dir: str, dtype: str, out_dir: str, max_tokens: int, lines: IO[
 def main(argv: Optional[List[str]] = None) -> int:
     args = build_parser().parse_args(argv)
     try:
-        return replay(args.model, args.dtype, args.out, args.max_tokens, sys.stdin, sys.stdout, device=args.device)
+        return replay(args.model, args.dtype, args.out, args.max_tokens, sys.stdin, sys.stdout, device=args.device,
+                      max_requests=args.max_requests)
     except Exception as error:      # one line on stderr, non-zero exit: the caller sees which step failed
         print(f"trace_run: {type(error).__name__}: {error}", file=sys.stderr, flush=True)
         return 1

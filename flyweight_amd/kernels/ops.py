@@ -19,7 +19,7 @@ from . import build as _build
 F32, BF16 = 0, 1
 PAGE_SIZE = 64          # tokens per cache page: the width of a wavefront
 MAX_HEAD_DIM = 256
-ABI_VERSION = 12
+ABI_VERSION = 13
 
 _lib = None
 
@@ -329,9 +329,10 @@ def qk_norm_rope_kv_write(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, 
                           cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], rotary_dim: int,
                           k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,
                           row_seg: torch.Tensor, row_pos: torch.Tensor, write_kv: bool = True,
-                          v_dim: Optional[int] = None) -> torch.Tensor:
+                          v_dim: Optional[int] = None, interleaved: bool = False) -> torch.Tensor:
     """The output and the cache take the pages' dtype; ``qkv`` may be float32 beside bfloat16 pages.
-    ``v_dim``: the size of a value head where it is not ``head_dim``."""
+    ``v_dim``: the size of a value head where it is not ``head_dim``. ``interleaved``: channel 2i turns
+    with channel 2i + 1 instead of channel i with channel i + rotary_dim / 2."""
     _dev(qkv, q_norm_weight, k_norm_weight, cos, sin, k_pages, v_pages, block_table, row_seg, row_pos)
     rows, width = qkv.shape
     v_dim = head_dim if v_dim is None else int(v_dim)
@@ -357,14 +358,17 @@ def qk_norm_rope_kv_write(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, 
     _check(library().fw_qk_norm_rope_kv_write(
         _p(qkv), _code(qkv.dtype), _p(q_out), _code(k_pages.dtype), _p(q_norm_weight), _p(k_norm_weight), ctypes.c_float(eps), _p(cos), _p(sin),
         rotary_dim, _p(k_pages), _p(v_pages), _p(block_table), block_table.shape[1], _p(row_seg), _p(row_pos), rows,
-        num_heads, num_kv_heads, head_dim, v_dim, PAGE_SIZE, pages, int(write_kv), _stream()))
+        num_heads, num_kv_heads, head_dim, v_dim, PAGE_SIZE, pages, int(write_kv), int(interleaved), _stream()))
     return q_out
 
 
 def attention_generic(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, k_pages: torch.Tensor,
                       v_pages: torch.Tensor, block_table: torch.Tensor, row_seg: torch.Tensor, row_pos: torch.Tensor,
-                      scale: float, window: int = 0, v_dim: Optional[int] = None) -> torch.Tensor:
-    """``v_dim``: the size of a value head (and of a head's output) where it is not ``head_dim``."""
+                      scale: float, window: int = 0, v_dim: Optional[int] = None, chunk: int = 0,
+                      softcap: float = 0.0) -> torch.Tensor:
+    """``v_dim``: the size of a value head (and of a head's output) where it is not ``head_dim``.
+    ``chunk`` > 0: a row sees only the keys of its own chunk of that many positions; ``softcap`` c > 0:
+    score <- c tanh(score / c)."""
     _dev(q, k_pages, v_pages, block_table, row_seg, row_pos)
     rows = q.shape[0]
     v_dim = head_dim if v_dim is None else int(v_dim)
@@ -379,8 +383,8 @@ def attention_generic(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
     out = torch.empty((rows, num_heads * v_dim), dtype=q.dtype, device=q.device)
     _check(library().fw_attention_generic(
         _p(q), _p(out), _code(q.dtype), _p(k_pages), _p(v_pages), _p(block_table), block_table.shape[1], _p(row_seg),
-        _p(row_pos), rows, num_heads, num_kv_heads, head_dim, v_dim, ctypes.c_float(scale), int(window), PAGE_SIZE, pages,
-        _stream()))
+        _p(row_pos), rows, num_heads, num_kv_heads, head_dim, v_dim, ctypes.c_float(scale), int(window), int(chunk),
+        ctypes.c_float(softcap), PAGE_SIZE, pages, _stream()))
     return out
 
 
@@ -874,18 +878,20 @@ def query_tiles(seg_row0):
     return tile_seg, tile_row0
 
 
-def decode_splits(max_context: int, window: int = 0) -> int:
+def decode_splits(max_context: int, window: int = 0, chunk: int = 0) -> int:
     """Into how many workgroups at most the keys that a row sees are cut: runs of 4 pages."""
     blocks = (max_context + PAGE_SIZE - 1) // PAGE_SIZE
-    if window > 0:
-        blocks = min(blocks, (window + PAGE_SIZE - 2) // PAGE_SIZE + 1)
+    span = min((n for n in (window, chunk) if n > 0), default=0)     # the most keys a row sees, where bounded
+    if span > 0:
+        blocks = min(blocks, (span + PAGE_SIZE - 2) // PAGE_SIZE + 1)
     return max(1, (blocks + DECODE_SPLIT_PAGES - 1) // DECODE_SPLIT_PAGES)
 
 
 def attention_prefill(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, k_pages: torch.Tensor,
                       v_pages: torch.Tensor, block_table: torch.Tensor, tile_seg: torch.Tensor, tile_row0: torch.Tensor,
                       seg_row0: torch.Tensor, row_pos: torch.Tensor, scale: float, window: int = 0,
-                      heads_together: int = 0, out: Optional[torch.Tensor] = None, v_dim: Optional[int] = None) -> torch.Tensor:
+                      heads_together: int = 0, out: Optional[torch.Tensor] = None, v_dim: Optional[int] = None,
+                      chunk: int = 0, softcap: float = 0.0) -> torch.Tensor:
     """``heads_together``: query heads of a kv group per workgroup (1, or 4 up to head_dim 64), 0: the
     kernel's choice. Only the rows of the given tiles are written (into ``out`` if given)."""
     _dev(q, k_pages, v_pages, block_table, tile_seg, tile_row0, seg_row0, row_pos)
@@ -907,7 +913,7 @@ def attention_prefill(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
     _check(library().fw_attention_prefill(
         _p(q), _p(out), _p(k_pages), _p(v_pages), _p(block_table), block_table.shape[1], _p(tile_seg), _p(tile_row0),
         tile_seg.numel(), _p(seg_row0), _p(row_pos), rows, num_heads, num_kv_heads, head_dim, v_dim, ctypes.c_float(scale),
-        int(window), PAGE_SIZE, pages, int(heads_together), _stream()))
+        int(window), int(chunk), ctypes.c_float(softcap), PAGE_SIZE, pages, int(heads_together), _stream()))
     return out
 
 
@@ -923,7 +929,8 @@ def _work(decode_work: Optional[torch.Tensor]):
 def attention_decode(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, k_pages: torch.Tensor,
                      v_pages: torch.Tensor, block_table: torch.Tensor, row_seg: torch.Tensor, row_pos: torch.Tensor,
                      scale: float, max_context: int, window: int = 0, out: Optional[torch.Tensor] = None,
-                     decode_work: Optional[torch.Tensor] = None, v_dim: Optional[int] = None) -> torch.Tensor:
+                     decode_work: Optional[torch.Tensor] = None, v_dim: Optional[int] = None, chunk: int = 0,
+                     softcap: float = 0.0) -> torch.Tensor:
     """One row per request; ``max_context`` bounds position + 1 of every row (the host knows it).
     ``decode_work``: one int32 on the device, the runs of 4 pages that the rows see together (the
     sum of ceil((position + 1) / 256)): the kernel shares the work out by it (fewer, longer
@@ -939,7 +946,7 @@ def attention_decode(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_di
         _want(t, torch.int32, name)
     if block_table.dim() != 2 or row_seg.numel() < rows or row_pos.numel() < rows:
         raise KernelError("attention: batch index arrays are too short")
-    splits = decode_splits(max_context, window)
+    splits = decode_splits(max_context, window, chunk)
     partial = torch.empty((rows, num_heads, splits, v_dim + 4), dtype=torch.float32, device=q.device)
     if out is None:
         out = torch.empty((rows, num_heads * v_dim), dtype=q.dtype, device=q.device)
@@ -951,7 +958,7 @@ def attention_decode(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_di
         _p(q), _p(out), _p(partial), splits, int(max_context), _work(decode_work), _p(tickets), tickets.numel(), _p(k_pages), _p(v_pages),
         _p(block_table),
         block_table.shape[1], _p(row_seg), _p(row_pos), rows, num_heads, num_kv_heads, head_dim, v_dim, ctypes.c_float(scale),
-        int(window), PAGE_SIZE, pages, _stream()))
+        int(window), int(chunk), ctypes.c_float(softcap), PAGE_SIZE, pages, _stream()))
     return out
 
 
@@ -960,7 +967,8 @@ def attention_decode_fused(qkv: torch.Tensor, num_heads: int, num_kv_heads: int,
                            cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], rotary_dim: int, k_pages: torch.Tensor,
                            v_pages: torch.Tensor, block_table: torch.Tensor, row_seg: torch.Tensor, row_pos: torch.Tensor,
                            scale: float, max_context: int, window: int = 0, write_kv: bool = True,
-                           decode_work: Optional[torch.Tensor] = None, v_dim: Optional[int] = None) -> torch.Tensor:
+                           decode_work: Optional[torch.Tensor] = None, v_dim: Optional[int] = None, chunk: int = 0,
+                           softcap: float = 0.0, interleaved: bool = False) -> torch.Tensor:
     """One row per request, from the step's raw projections ``qkv`` (float32 [rows, (heads + 2 kv
     heads) * head_dim]): per-head norm and rotation of queries and keys, the new keys and values
     into their pages, and the split-key attention, in one kernel. Returns bfloat16 [rows, heads *
@@ -986,7 +994,7 @@ def attention_decode_fused(qkv: torch.Tensor, num_heads: int, num_kv_heads: int,
         _want(t, torch.int32, name)
     if block_table.dim() != 2 or row_seg.numel() < rows or row_pos.numel() < rows:
         raise KernelError("attention: batch index arrays are too short")
-    splits = decode_splits(max_context, window)
+    splits = decode_splits(max_context, window, chunk)
     partial = torch.empty((rows, num_heads, splits, v_dim + 4), dtype=torch.float32, device=qkv.device)
     out = torch.empty((rows, num_heads * v_dim), dtype=torch.bfloat16, device=qkv.device)
     group = num_heads // num_kv_heads
@@ -995,7 +1003,7 @@ def attention_decode_fused(qkv: torch.Tensor, num_heads: int, num_kv_heads: int,
         _p(qkv), _p(q_norm_weight), _p(k_norm_weight), ctypes.c_float(eps), _p(cos), _p(sin), int(rotary_dim), int(write_kv), _p(out),
         _p(partial), splits, int(max_context), _work(decode_work), _p(tickets), tickets.numel(), _p(k_pages), _p(v_pages), _p(block_table),
         block_table.shape[1], _p(row_seg), _p(row_pos), rows, num_heads, num_kv_heads, head_dim, v_dim, ctypes.c_float(scale), int(window),
-        PAGE_SIZE, pages, _stream()))
+        int(chunk), ctypes.c_float(softcap), int(interleaved), PAGE_SIZE, pages, _stream()))
     return out
 
 
@@ -1008,7 +1016,8 @@ def attention_is_tiled(head_dim: int) -> bool:
 def attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, k_pages: torch.Tensor,
               v_pages: torch.Tensor, block_table: torch.Tensor, ctx, scale: float, window: int = 0,
               tile_seg: Optional[torch.Tensor] = None, tile_row0: Optional[torch.Tensor] = None,
-              decode_work: Optional[torch.Tensor] = None, v_dim: Optional[int] = None) -> torch.Tensor:
+              decode_work: Optional[torch.Tensor] = None, v_dim: Optional[int] = None, chunk: int = 0,
+              softcap: float = 0.0) -> torch.Tensor:
     """bfloat16 with a head size in steps of 16 runs on the matrix cores: the split-key decode
     kernel for segments of one row (all of them, or those a mixed step begins with: a single row
     would hold a 64-row tile of the prompt kernel and walk its whole context alone), the tiled
@@ -1020,7 +1029,8 @@ def attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
     fast = q.dtype == torch.bfloat16 and attention_is_tiled(head_dim) and attention_is_tiled(v_dim)
     if fast and ctx.all_decode:
         return attention_decode(q, num_heads, num_kv_heads, head_dim, k_pages, v_pages, block_table, ctx.row_seg,
-                                ctx.row_pos, scale, ctx.max_context, window, decode_work=decode_work, v_dim=v_dim)
+                                ctx.row_pos, scale, ctx.max_context, window, decode_work=decode_work, v_dim=v_dim,
+                                chunk=chunk, softcap=softcap)
     if fast:
         if tile_seg is None or tile_row0 is None:
             raise KernelError("attention: the tiled kernel needs the step's query tiles")
@@ -1029,30 +1039,34 @@ def attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
         # (a page is read once for the four); from the start of a prompt one head per workgroup
         # gives more and shorter workgroups, which evens out the causal triangle
         rows = q.shape[0] - single
-        keys = min(window, ctx.max_context) if window else ctx.max_context      # the most keys a row can see
+        keys = min([n for n in (window, chunk) if n] + [ctx.max_context])      # the most keys a row can see
         together = 4 if max(head_dim, v_dim) <= 64 and num_heads // num_kv_heads >= 4 and keys >= 4 * rows else 0
         if single == 0:
             return attention_prefill(q, num_heads, num_kv_heads, head_dim, k_pages, v_pages, block_table, tile_seg,
-                                     tile_row0, ctx.seg_row0, ctx.row_pos, scale, window, heads_together=together, v_dim=v_dim)
+                                     tile_row0, ctx.seg_row0, ctx.row_pos, scale, window, heads_together=together, v_dim=v_dim,
+                                     chunk=chunk, softcap=softcap)
         out = torch.empty((q.shape[0], num_heads * v_dim), dtype=q.dtype, device=q.device)
         attention_decode(q[:single], num_heads, num_kv_heads, head_dim, k_pages, v_pages, block_table, ctx.row_seg,
-                         ctx.row_pos, scale, ctx.max_context, window, out=out[:single], decode_work=decode_work, v_dim=v_dim)
+                         ctx.row_pos, scale, ctx.max_context, window, out=out[:single], decode_work=decode_work, v_dim=v_dim,
+                         chunk=chunk, softcap=softcap)
         return attention_prefill(q, num_heads, num_kv_heads, head_dim, k_pages, v_pages, block_table,
                                  tile_seg[single:], tile_row0[single:], ctx.seg_row0, ctx.row_pos, scale, window,
-                                 heads_together=together, out=out, v_dim=v_dim)
+                                 heads_together=together, out=out, v_dim=v_dim, chunk=chunk, softcap=softcap)
     return attention_generic(q, num_heads, num_kv_heads, head_dim, k_pages, v_pages, block_table, ctx.row_seg,
-                             ctx.row_pos, scale, window, v_dim=v_dim)
+                             ctx.row_pos, scale, window, v_dim=v_dim, chunk=chunk, softcap=softcap)
 
 
 # ---- the gated delta rule -----------------------------------------------------------------------------
 def delta_prepare(proj: torch.Tensor, beta_col: int, a: torch.Tensor, taps: torch.Tensor, conv_state: torch.Tensor,
                   A_log: torch.Tensor, dt_bias: torch.Tensor, row_seg: torch.Tensor, seg_row0: torch.Tensor,
-                  seg_slot: torch.Tensor, segments: int, heads: int, kv_heads: int, dim: int, vdim: int):
+                  seg_slot: torch.Tensor, segments: int, heads: int, kv_heads: int, dim: int, vdim: int,
+                  decay_per_head: bool = False):
     """From a step's projections to what the recurrence reads. ``proj`` [rows, >= channels + ...]:
     its first ``channels`` = 2 kv_heads dim + heads vdim columns are q | k | v before their short
     convolutions, columns ``beta_col`` .. + heads the write strengths before the sigmoid; ``a``
     [rows, heads dim] the decays' arguments. ``conv_state`` [slots, channels, taps - 1] is read and
-    moved on. Returns float32 records [rows, heads, delta_record_floats(dim, vdim)]: per row and head
+    moved on. ``decay_per_head``: one decay for all key channels of a head (``a`` [rows, heads],
+    ``dt_bias`` [heads]). Returns float32 records [rows, heads, delta_record_floats(dim, vdim)]: per row and head
     q | k | g | beta | v as the recurrence reads them (q and k of the head's group)."""
     _dev(proj, taps, conv_state, A_log, dt_bias, row_seg, seg_row0, seg_slot)
     _dev_rows(a, "a")
@@ -1061,9 +1075,10 @@ def delta_prepare(proj: torch.Tensor, beta_col: int, a: torch.Tensor, taps: torc
     count = taps.shape[1]
     if proj.dtype != a.dtype or not proj.is_contiguous() or a.dim() != 2 or a.stride(1) != 1:
         raise KernelError("delta_prepare: the projections and the decays' arguments come in one dtype, rows contiguous")
-    if a.shape != (rows, heads * dim):
-        raise KernelError(f"delta_prepare: a is {tuple(a.shape)}, expected {(rows, heads * dim)} (a view of wider rows will do)")
-    for name, t, shape in (("taps", taps, (channels, count)), ("A_log", A_log, (heads,)), ("dt_bias", dt_bias, (heads * dim,))):
+    decays = heads if decay_per_head else heads * dim
+    if a.shape != (rows, decays):
+        raise KernelError(f"delta_prepare: a is {tuple(a.shape)}, expected {(rows, decays)} (a view of wider rows will do)")
+    for name, t, shape in (("taps", taps, (channels, count)), ("A_log", A_log, (heads,)), ("dt_bias", dt_bias, (decays,))):
         _want(t, torch.float32, name)
         if t.shape != shape or not t.is_contiguous():
             raise KernelError(f"delta_prepare: {name} is {tuple(t.shape)}, expected {shape}")
@@ -1075,9 +1090,10 @@ def delta_prepare(proj: torch.Tensor, beta_col: int, a: torch.Tensor, taps: torc
         if t.numel() < n:
             raise KernelError(f"delta_prepare: {name} holds {t.numel()} entries, needs {n}")
     records = torch.empty((rows, heads, delta_record_floats(dim, vdim)), dtype=torch.float32, device=proj.device)
-    _check(library().fw_delta_prepare(_p(proj), _code(proj.dtype), stride, int(beta_col), _p(a), a.stride(0) if rows > 1 else heads * dim,
+    _check(library().fw_delta_prepare(_p(proj), _code(proj.dtype), stride, int(beta_col), _p(a), a.stride(0) if rows > 1 else max(decays, a.stride(0)),
                                       _p(taps), _p(conv_state), _p(A_log), _p(dt_bias), _p(row_seg), _p(seg_row0), _p(seg_slot),
-                                      _p(records), rows, int(segments), heads, kv_heads, dim, vdim, count, conv_state.shape[0], _stream()))
+                                      _p(records), rows, int(segments), heads, kv_heads, dim, vdim, count, conv_state.shape[0],
+                                      int(decay_per_head), _stream()))
     return records
 
 
@@ -1111,8 +1127,8 @@ def gated_delta_rule(records: torch.Tensor, state: torch.Tensor, seg_row0: torch
 
 
 def gated_head_norm(o: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, heads: int, vdim: int, eps: float,
-                    out_dtype: torch.dtype) -> torch.Tensor:
-    """Per head: o / rms(o) * weight * sigmoid(gate); ``o`` float32 [rows, heads vdim], ``gate``
+                    out_dtype: torch.dtype, gate_silu: bool = False) -> torch.Tensor:
+    """Per head: o / rms(o) * weight * sigmoid(gate) (``gate_silu``: times gate * sigmoid(gate)); ``o`` float32 [rows, heads vdim], ``gate``
     [rows, heads vdim] (float32, or bfloat16 beside a bfloat16 output; a view of wider rows will do)."""
     _dev(o, weight)
     _dev_rows(gate, "gate")
@@ -1122,8 +1138,8 @@ def gated_head_norm(o: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, h
     if o.shape != (rows, heads * vdim) or gate.shape != o.shape or weight.shape != (vdim,) or not o.is_contiguous() or gate.stride(1) != 1:
         raise KernelError(f"gated_head_norm: o {tuple(o.shape)}, gate {tuple(gate.shape)}, weight {tuple(weight.shape)} do not fit {heads} x {vdim}")
     out = torch.empty((rows, heads * vdim), dtype=out_dtype, device=o.device)
-    _check(library().fw_gated_head_norm(_p(o), _p(gate), _code(gate.dtype), gate.stride(0) if rows > 1 else heads * vdim, _p(weight), _p(out), _code(out_dtype), rows,
-                                        heads, vdim, ctypes.c_float(eps), _stream()))
+    _check(library().fw_gated_head_norm(_p(o), _p(gate), _code(gate.dtype), gate.stride(0) if rows > 1 else max(heads * vdim, gate.stride(0)), _p(weight), _p(out), _code(out_dtype), rows,
+                                        heads, vdim, ctypes.c_float(eps), int(gate_silu), _stream()))
     return out
 
 
@@ -1170,4 +1186,119 @@ def clamped_glu(gate_up: torch.Tensor, limit: float, alpha: float, shift: float,
     out = torch.empty((rows, width // 2), dtype=out_dtype, device=gate_up.device)
     _check(library().fw_clamped_glu(_p(gate_up), _code(gate_up.dtype), _p(out), _code(out_dtype), rows, width // 2,
                                     ctypes.c_float(limit), ctypes.c_float(alpha), ctypes.c_float(shift), _stream()))
+    return out
+
+
+# ---- a sublayer between two norms, layer norm, the gate on a second token table ------------------------------
+NEXT_NOTHING, NEXT_ROUNDED, NEXT_RMS, NEXT_CENTERED = 0, 1, 2, 3
+
+
+def layernorm_rows(x: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch.dtype,
+                   row_index: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """(x - mean) / sqrt(mean((x - mean)^2) + eps) * weight over float32 rows (gathered through
+    ``row_index`` if given), in ``out_dtype``."""
+    _dev(x, weight, row_index)
+    _want(x, torch.float32, "x")
+    _want(weight, torch.float32, "weight")
+    hidden = x.shape[-1]
+    if weight.shape != (hidden,):
+        raise KernelError(f"layernorm: weight is {tuple(weight.shape)}, row width is {hidden}")
+    rows = x.numel() // hidden if row_index is None else row_index.numel()
+    if row_index is not None:
+        _want(row_index, torch.int32, "row_index")
+    out = torch.empty((rows, hidden), dtype=out_dtype, device=x.device)
+    _check(library().fw_layernorm_rows(_p(x), _p(weight), _p(out), _code(out_dtype), _p(row_index), rows, hidden,
+                                       ctypes.c_float(eps), _stream()))
+    return out
+
+
+def norm_add_norm_(x: torch.Tensor, a: torch.Tensor, weight: torch.Tensor, centered: bool, eps: float, *,
+                   next_kind: int = NEXT_NOTHING, next_weight: Optional[torch.Tensor] = None, next_eps: float = 0.0,
+                   next_dtype: Optional[torch.dtype] = None) -> Optional[torch.Tensor]:
+    """x += norm(a) * weight in place (float32 rows; ``centered``: the row's mean is taken off before its
+    root mean square). What reads x next is formed from the new rows in the same kernel and returned:
+    ``NEXT_ROUNDED`` the rows in ``next_dtype``, ``NEXT_RMS`` / ``NEXT_CENTERED`` their norm with
+    ``next_weight`` and ``next_eps``; ``NEXT_NOTHING`` returns None."""
+    _dev(x, a, weight, next_weight)
+    rows, hidden = x.shape
+    for name, t in (("x", x), ("a", a)):
+        _want(t, torch.float32, name)
+        if t.shape != (rows, hidden):
+            raise KernelError(f"norm_add_norm: {name} is {tuple(t.shape)}, expected {(rows, hidden)}")
+    for name, t in (("weight", weight), ("next_weight", next_weight)):
+        if t is not None:
+            _want(t, torch.float32, name)
+            if t.shape != (hidden,):
+                raise KernelError(f"norm_add_norm: {name} is {tuple(t.shape)}, row width is {hidden}")
+    if next_kind not in (NEXT_NOTHING, NEXT_ROUNDED, NEXT_RMS, NEXT_CENTERED):
+        raise KernelError(f"norm_add_norm: unknown kind {next_kind} of what follows")
+    if next_kind >= NEXT_RMS and next_weight is None:
+        raise KernelError("norm_add_norm: the norm that follows needs its weight")
+    out = None
+    if next_kind != NEXT_NOTHING:
+        out = torch.empty((rows, hidden), dtype=next_dtype or torch.float32, device=x.device)
+    _check(library().fw_norm_add_norm(_p(x), _p(a), _p(weight), int(centered), ctypes.c_float(eps), int(next_kind), _p(next_weight),
+                                      ctypes.c_float(next_eps), _p(out), _code(out.dtype) if out is not None else F32, rows, hidden,
+                                      _stream()))
+    return out
+
+
+def gelu_gate_rows(z: torch.Tensor, table: torch.Tensor, ids: torch.Tensor, col0: int, out_dtype: torch.dtype) -> torch.Tensor:
+    """gelu_tanh(z) * table[ids][:, col0 : col0 + width]: ``z`` float32 [rows, width], ``table`` [entries,
+    columns], ``ids`` int32 [rows] (checked against the table by the caller)."""
+    _dev(z, table, ids)
+    _want(z, torch.float32, "z")
+    _want(ids, torch.int32, "ids")
+    rows, width = z.shape
+    if table.dim() != 2 or col0 < 0 or col0 + width > table.shape[1] or ids.numel() < rows:
+        raise KernelError(f"gelu_gate_rows: columns {col0}..{col0 + width} of a table {tuple(table.shape)}, {ids.numel()} ids for {rows} rows")
+    out = torch.empty((rows, width), dtype=out_dtype, device=z.device)
+    _check(library().fw_gelu_gate_rows(_p(z), width, _p(table), _code(table.dtype), table.shape[0], table.shape[1], int(col0), _p(ids),
+                                       _p(out), _code(out_dtype), rows, width, _stream()))
+    return out
+
+
+# ---- attention over a cached latent ------------------------------------------------------------------------
+def latent_norm_write(raw: torch.Tensor, weight: torch.Tensor, eps: float, k_pages: torch.Tensor, v_pages: torch.Tensor,
+                      block_table: torch.Tensor, row_seg: torch.Tensor, row_pos: torch.Tensor) -> None:
+    """The step's latents ``raw`` (float32 [rows, rank]; a view of some columns of wider rows will do), RMS-normed
+    times ``weight``, stored at each row's position in a cache of one key/value head of ``rank`` channels."""
+    _dev(weight, k_pages, v_pages, block_table, row_seg, row_pos)
+    _dev_rows(raw, "raw")
+    _want(raw, torch.float32, "raw")
+    _want(weight, torch.float32, "weight")
+    rows, rank = raw.shape
+    if weight.shape != (rank,):
+        raise KernelError(f"latent_norm_write: weight is {tuple(weight.shape)}, the latent has {rank} channels")
+    pages = _check_pages(k_pages, v_pages, 1, rank, k_pages.dtype, rank)
+    for name, t in (("block_table", block_table), ("row_seg", row_seg), ("row_pos", row_pos)):
+        _want(t, torch.int32, name)
+    if block_table.dim() != 2 or row_seg.numel() < rows or row_pos.numel() < rows:
+        raise KernelError("latent_norm_write: batch index arrays are too short")
+    _check(library().fw_latent_norm_write(_p(raw), raw.stride(0) if rows > 1 else max(rank, raw.stride(0)), 0, _p(weight), ctypes.c_float(eps),
+                                          _p(k_pages), _p(v_pages), _code(k_pages.dtype), _p(block_table), block_table.shape[1],
+                                          _p(row_seg), _p(row_pos), rows, rank, PAGE_SIZE, pages, _stream()))
+
+
+def head_linear(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """A map per head: ``x`` [rows, heads K] (rows may lie apart), ``w`` [heads, N, K] -> [rows, heads N], with
+    ``gate`` (float32 [rows, heads N], rows may lie apart) times its sigmoid."""
+    _dev(w)
+    _dev_rows(x, "x")
+    heads, N, K = w.shape
+    rows = x.shape[0]
+    if x.shape[1] != heads * K:
+        raise KernelError(f"head_linear: x is {tuple(x.shape)}, the weight {tuple(w.shape)}")
+    if gate is not None:
+        _dev_rows(gate, "gate")
+        if gate.shape != (rows, heads * N) or gate.dtype != torch.float32:
+            raise KernelError(f"head_linear: the gate is {tuple(gate.shape)} {gate.dtype}, expected {(rows, heads * N)} float32")
+    out = torch.empty((rows, heads * N), dtype=out_dtype, device=x.device)
+
+    def stride(t: torch.Tensor, width: int) -> int:
+        return t.stride(0) if rows > 1 else max(width, t.stride(0))
+
+    _check(library().fw_head_linear(_p(x), _code(x.dtype), stride(x, heads * K), _p(w), _code(w.dtype), _p(gate),
+                                    stride(gate, heads * N) if gate is not None else 0, _p(out), _code(out_dtype), rows, heads, N, K,
+                                    _stream()))
     return out

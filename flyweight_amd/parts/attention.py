@@ -3,8 +3,9 @@
 q = W_q h, k = W_k h, v = W_v h; optional per-head RMS norm of q and k (one weight of
 head_dim shared by all heads); position encoding on q and k; k and v appended to the
 cache; scores q.k * softmax_scale (1 / sqrt(head_dim) unless given) over the cached keys the row
-may see (causal, optionally only the last ``window``: itself and the window - 1 before it),
-softmax in float32, weighted sum of values; out = W_o o. Values may have a size of their own
+may see (causal, optionally only the last ``window``: itself and the window - 1 before it; with
+``chunk`` only those of the row's own chunk of that many positions, chunks counted from position 0 of
+the sequence), optionally capped softly (``score_softcap`` c: c tanh(score / c)), softmax in float32, weighted sum of values; out = W_o o. Values may have a size of their own
 (``v_head_dim``); the output of a head has that size.
 Query head i reads kv head i // (num_heads / num_kv_heads). Formulas as the reference's
 LFM2 attention branch computes them (native/src/v2_runtime.cpp:28429-28478).
@@ -46,6 +47,8 @@ class GQAttention(Mixer):
         self.qk_norm = bool(spec.get("qk_norm", False))
         self.qk_norm_eps = float(spec.get("qk_norm_eps", 1e-6)) if self.qk_norm else 1.0
         self.window = spec.get("window")
+        self.chunk = int(spec.get("chunk") or 0)
+        self.softcap = float(spec.get("score_softcap") or 0.0)
         self.scale = float(spec.get("softmax_scale", self.head_dim ** -0.5))
         self.bias = bool(spec.get("bias", False))
         self.names = {**_DEFAULT_NAMES, **dict(spec.get("names", {}))}
@@ -60,6 +63,8 @@ class GQAttention(Mixer):
             raise ConfigError("biases need the '.weight' / '.bias' tensor names")
         if self.window is not None and int(self.window) <= 0:
             raise ConfigError("an attention window must be positive (or None for all keys)")
+        if self.chunk < 0 or self.softcap < 0:
+            raise ConfigError("an attention chunk and a soft cap on the scores must be positive (or 0 / None for none)")
 
     def cache_need(self):
         return PagedKV(self.num_kv_heads, self.head_dim, None if self.window is None else int(self.window),
@@ -142,6 +147,7 @@ class GQAttention(Mixer):
         values appended to the cache on the way."""
         qkv = self.qkv.forward(h, out_dtype=torch.float32)      # normed, rotated and rounded once, below
         cos, sin = ctx.position_tables(self.position)
+        interleaved = bool(getattr(self.position, "interleaved", False))
         own = ctx.step_arrays(self) if self.step_arrays_key() is not None else {}
         if ctx.all_decode and ctx.num_rows <= self.FUSED_DECODE_ROWS and qkv.dtype == torch.float32 and self.step_arrays_key() is not None:
             # a few single-token segments on the matrix cores: norm, rotation, cache write and attention in one kernel
@@ -149,15 +155,16 @@ class GQAttention(Mixer):
                 qkv, self.num_heads, self.num_kv_heads, self.head_dim, self.q_norm_weight, self.k_norm_weight, self.qk_norm_eps,
                 cos, sin, self.position.rotary_dim, cache.k_pages, cache.v_pages, cache.block_table, ctx.row_seg, ctx.row_pos,
                 self.scale, ctx.max_context, int(self.window or 0), write_kv=cache.writes,
-                decode_work=own.get("decode_work"), v_dim=self.v_head_dim)
+                decode_work=own.get("decode_work"), v_dim=self.v_head_dim, chunk=self.chunk, softcap=self.softcap,
+                interleaved=interleaved)
         q = ops.qk_norm_rope_kv_write(
             qkv, self.num_heads, self.num_kv_heads, self.head_dim, self.q_norm_weight, self.k_norm_weight,
             self.qk_norm_eps, cos, sin, self.position.rotary_dim, cache.k_pages, cache.v_pages, cache.block_table,
-            ctx.row_seg, ctx.row_pos, write_kv=cache.writes, v_dim=self.v_head_dim)
+            ctx.row_seg, ctx.row_pos, write_kv=cache.writes, v_dim=self.v_head_dim, interleaved=interleaved)
         return ops.attention(q, self.num_heads, self.num_kv_heads, self.head_dim, cache.k_pages, cache.v_pages,
                              cache.block_table, ctx, self.scale, int(self.window or 0),
                              tile_seg=own.get("tile_seg"), tile_row0=own.get("tile_row0"), decode_work=own.get("decode_work"),
-                             v_dim=self.v_head_dim)
+                             v_dim=self.v_head_dim, chunk=self.chunk, softcap=self.softcap)
 
     def forward(self, h, residual, ctx, cache):
         return self.out.accumulate(self.attend(h, ctx, cache), residual, then=getattr(ctx, "upcoming_norm", None))

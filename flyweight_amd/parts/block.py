@@ -7,6 +7,11 @@ arrangement (post-norm, parallel mixer and feed-forward) is another class regist
 ``output_norm_residual``: x <- x + m * norm1(mixer(x)); x <- x + m * norm2(ffn(x)). The sublayers
 read x itself (rounded to the activation dtype for their products), the norm stands on a
 sublayer's OUTPUT, and m is a fixed factor. The feed-forward may be absent.
+
+``sandwich_norm_residual``: x <- x + post1(mixer(pre1(x))); x <- x + post2(ffn(pre2(x))), a norm before
+and a norm behind every sublayer; then, where the layer has one, the tokens' own input
+(``parts/token_input.py``): x <- x + rms(y(x, token)) * w. The feed-forward may be absent. Every sum into
+x also forms what reads x next (the next norm's output, or x rounded) in the same kernel.
 """
 
 from __future__ import annotations
@@ -14,7 +19,8 @@ from __future__ import annotations
 from ..config.spec import ConfigError
 from ..kernels import ops
 from .base import Block, build_part, register_block
-from .norm import LazyNorm
+from .norm import LazyNorm, NormedRows
+from .token_input import TokenInput
 
 
 @register_block("pre_norm_residual")
@@ -122,3 +128,70 @@ class OutputNormResidualBlock(Block):
             h = x if rounded is None else rounded
             rounded = self._join(x, self._terms(self.ffn, h, ctx), self.ffn_norm, dtype)
         return None if rounded is None else RoundedRows(rounded)
+
+
+@register_block("sandwich_norm_residual")
+class SandwichNormResidualBlock(Block):
+    """``LayerSpec.params``: ``mixer_post_norm`` and ``ffn_post_norm`` (PartSpecs of norms), ``token_input``
+    (PartSpec of a :class:`TokenInput`, or absent). The norms may be RMS or layer norms, each on its own."""
+
+    def __init__(self, spec):
+        self.spec = spec
+        self.mixer_norm = build_part("norm", spec.mixer_norm)
+        self.mixer = build_part("mixer", spec.mixer)
+        self.mixer_post_norm = build_part("norm", spec.params["mixer_post_norm"])
+        self.ffn = build_part("ffn", spec.ffn) if spec.ffn is not None else None
+        self.ffn_norm = build_part("norm", spec.ffn_norm) if spec.ffn is not None else None
+        self.ffn_post_norm = build_part("norm", spec.params["ffn_post_norm"]) if spec.ffn is not None else None
+        given = spec.params.get("token_input")
+        self.token_input = TokenInput(given) if given is not None else None
+        for part in (self.mixer, self.ffn):
+            if part is not None and not hasattr(part, "output"):
+                raise ConfigError(f"part '{part.spec.kind}' cannot give its output apart from the residual stream")
+        for norm in (self.mixer_norm, self.mixer_post_norm, self.ffn_norm, self.ffn_post_norm):
+            if norm is not None and (not hasattr(norm, "row_norm") or getattr(norm, "one_centered", False)):
+                raise ConfigError("the sandwich arrangement takes RMS norms with a plain weight and layer norms")
+
+    def parts(self):
+        return tuple(part for part in (self.mixer_norm, self.mixer, self.mixer_post_norm, self.ffn_norm, self.ffn,
+                                       self.ffn_post_norm, self.token_input) if part is not None)
+
+    def first_norm(self):
+        return self.mixer_norm
+
+    def cache_need(self):
+        return self.mixer.cache_need()
+
+    @property
+    def graph_safe(self) -> bool:
+        position = getattr(self.mixer, "position", None)
+        return all(part.graph_safe for part in self.parts()) and (position is None or position.graph_safe)
+
+    def _join(self, x, rows, norm, reader, dtype):
+        """x += norm(rows); returns what ``reader`` sees of the new x: a norm's output (``reader`` a norm),
+        x rounded (``reader`` "rounded"), or None (``reader`` None)."""
+        weight, eps, centered = norm.row_norm()
+        if reader is None:
+            ops.norm_add_norm_(x, rows, weight, centered, eps)
+            return None
+        if reader == "rounded":
+            return ops.norm_add_norm_(x, rows, weight, centered, eps, next_kind=ops.NEXT_ROUNDED, next_dtype=dtype)
+        next_weight, next_eps, next_centered = reader.row_norm()
+        return ops.norm_add_norm_(x, rows, weight, centered, eps, next_kind=ops.NEXT_CENTERED if next_centered else ops.NEXT_RMS,
+                                  next_weight=next_weight, next_eps=next_eps, next_dtype=dtype)
+
+    def forward(self, x, ctx, cache, prepared=None, norm_after=None):
+        """``x`` [rows, hidden] float32 is updated in place."""
+        dtype = self.mixer_norm.dtype
+        # a norm that follows this block is formed with the block's last sum only if it is of a form the kernel knows
+        after = norm_after if hasattr(norm_after, "row_norm") and norm_after.row_norm() is not None else None
+        h = LazyNorm(self.mixer_norm, x, ctx, prepared=prepared).tensor()
+        last = self.ffn is None and self.token_input is None
+        reader = after if last else (self.ffn_norm if self.ffn is not None else "rounded")
+        h = self._join(x, self.mixer.output(h, ctx, cache), self.mixer_post_norm, reader, dtype)
+        if self.ffn is not None:
+            reader = after if self.token_input is None else "rounded"
+            h = self._join(x, self.ffn.output(h, ctx), self.ffn_post_norm, reader, dtype)
+        if self.token_input is not None:
+            h = self._join(x, self.token_input.output(h, ctx), self.token_input, after, dtype)
+        return NormedRows(after, h) if after is not None and h is not None else None

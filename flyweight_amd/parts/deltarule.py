@@ -12,6 +12,11 @@ sigmoid(W_b h) and a decay per key channel g = exp(-exp(A_log) * softplus(W_a2 W
 a weight of vdim shared by the heads, times sigmoid(W_g2 W_g1 h); out = W_o of the heads side by
 side. The state S and everything that enters the recurrence besides the projections is float32.
 A request keeps S (zero at the start) and the convolutions' last taps - 1 inputs.
+
+Two parameters choose between forms of the decay and of the output gate. ``decay`` "channel_low_rank" (the
+default) is the above; "head" is one decay for all key channels of a head, g = exp(-exp(A_log) *
+softplus(W_a h + dt_bias)) with W_a [heads, hidden] and dt_bias [heads]. ``gate`` "low_rank_sigmoid" (the
+default) is the above; "silu" multiplies by silu(W_g h) with W_g [heads vdim, hidden].
 """
 
 from __future__ import annotations
@@ -27,7 +32,7 @@ from ..weights.loader import TensorDecl
 from .base import Mixer, register_mixer
 from .linear import Linear
 
-_DEFAULT_NAMES = {"q": "q", "k": "k", "v": "v", "b": "b", "a1": "a1", "a2": "a2", "g1": "g1", "g2": "g2", "o": "o",
+_DEFAULT_NAMES = {"q": "q", "k": "k", "v": "v", "b": "b", "a": "a", "a1": "a1", "a2": "a2", "g": "g", "g1": "g1", "g2": "g2", "o": "o",
                   "q_conv": "q.conv", "k_conv": "k.conv", "v_conv": "v.conv", "A_log": "A_log", "dt_bias": "dt_bias",
                   "norm": "norm"}
 
@@ -44,8 +49,12 @@ class GatedDeltaRule(Mixer):
         self.dim = int(spec["head_dim"])
         self.vdim = int(spec["v_head_dim"])
         self.taps_count = int(spec["conv_taps"])
-        self.rank_a = int(spec["decay_rank"])
-        self.rank_g = int(spec["gate_rank"])
+        self.decay = str(spec.get("decay", "channel_low_rank"))
+        self.gate = str(spec.get("gate", "low_rank_sigmoid"))
+        if self.decay not in ("channel_low_rank", "head") or self.gate not in ("low_rank_sigmoid", "silu"):
+            raise ConfigError(f"gated delta rule: unknown form of the decay '{self.decay}' or of the gate '{self.gate}'")
+        self.rank_a = int(spec["decay_rank"]) if self.decay == "channel_low_rank" else 0
+        self.rank_g = int(spec["gate_rank"]) if self.gate == "low_rank_sigmoid" else 0
         self.eps = float(spec["norm_eps"])
         self.names = {**_DEFAULT_NAMES, **dict(spec.get("names", {}))}
         if self.heads % self.kv_heads:
@@ -72,34 +81,60 @@ class GatedDeltaRule(Mixer):
 
     def tensors(self) -> Dict[str, TensorDecl]:
         D, H, G, d, dv, L = self.hidden, self.heads, self.kv_heads, self.dim, self.vdim, self.taps_count
-        return {
+        declared = {
             self._name("q"): TensorDecl((G * d, D)), self._name("k"): TensorDecl((G * d, D)), self._name("v"): TensorDecl((H * dv, D)),
             self._name("q_conv"): TensorDecl((G * d, L), "vector", "conv"), self._name("k_conv"): TensorDecl((G * d, L), "vector", "conv"),
             self._name("v_conv"): TensorDecl((H * dv, L), "vector", "conv"),
             self._name("b"): TensorDecl((H, D)), self._name("A_log"): TensorDecl((H,), "vector", "bias"),
             self._name("norm"): TensorDecl((dv,), "vector", "norm"),
-            self._name("a1"): TensorDecl((self.rank_a, D)), self._name("a2"): TensorDecl((H * d, self.rank_a)),
-            self._name("dt_bias"): TensorDecl((H * d,), "vector", "bias"),
-            self._name("g1"): TensorDecl((self.rank_g, D)), self._name("g2"): TensorDecl((H * dv, self.rank_g)),
             self._name("o"): TensorDecl((D, H * dv)),
         }
+        if self.decay == "head":
+            declared[self._name("a")] = TensorDecl((H, D))
+            declared[self._name("dt_bias")] = TensorDecl((H,), "vector", "bias")
+        else:
+            declared[self._name("a1")] = TensorDecl((self.rank_a, D))
+            declared[self._name("a2")] = TensorDecl((H * d, self.rank_a))
+            declared[self._name("dt_bias")] = TensorDecl((H * d,), "vector", "bias")
+        if self.gate == "silu":
+            declared[self._name("g")] = TensorDecl((H * dv, D))
+        else:
+            declared[self._name("g1")] = TensorDecl((self.rank_g, D))
+            declared[self._name("g2")] = TensorDecl((H * dv, self.rank_g))
+        return declared
 
     def bind(self, tensors, dtype, device) -> None:
         super().bind(tensors, dtype, device)
-        t = {which: tensors[self._name(which)] for which in self.names}
+        t = {which: tensors[self._name(which)] for which in self.names if self._name(which) in self.tensors()}
         # One operand for what the recurrence reads of h in float32: q | k | v (the convolutions' inputs)
         # and the write strengths. The two low-rank maps share their two products: the inner halves
         # side by side (their activations leave in the activation dtype, as any product's input), and
         # the outer halves as one block-diagonal operand whose zeros add nothing, so that one product
         # gives the decays' arguments and the gates side by side.
         self.beta_col = self.channels
-        self.in_proj = Linear(torch.cat([t["q"], t["k"], t["v"], t["b"]], dim=0))
-        self.low = Linear(torch.cat([t["a1"], t["g1"]], dim=0))
-        a2, g2 = t["a2"], t["g2"]
-        outer = torch.zeros((a2.shape[0] + g2.shape[0], self.rank_a + self.rank_g), dtype=a2.dtype, device=a2.device)
-        outer[:a2.shape[0], :self.rank_a] = a2
-        outer[a2.shape[0]:, self.rank_a:] = g2
-        self.outer = Linear(outer)
+        # Maps that read h directly (a decay per head, a full-rank gate) join that operand: the decays'
+        # arguments behind the write strengths, the gates behind them, all float32 sums of one product.
+        direct = [t["q"], t["k"], t["v"], t["b"]]
+        self.a_col = self.gate_col = None
+        if self.decay == "head":
+            self.a_col = sum(m.shape[0] for m in direct)
+            direct.append(t["a"])
+        if self.gate == "silu":
+            self.gate_col = sum(m.shape[0] for m in direct)
+            direct.append(t["g"])
+        self.in_proj = Linear(torch.cat(direct, dim=0))
+        inner = ([t["a1"]] if self.decay != "head" else []) + ([t["g1"]] if self.gate != "silu" else [])
+        self.low = self.outer = None
+        if inner:
+            self.low = Linear(torch.cat(inner, dim=0))
+            blocks = ([t["a2"]] if self.decay != "head" else []) + ([t["g2"]] if self.gate != "silu" else [])
+            outer = torch.zeros((sum(b.shape[0] for b in blocks), sum(b.shape[1] for b in blocks)), dtype=blocks[0].dtype,
+                                device=blocks[0].device)
+            row = col = 0
+            for b in blocks:
+                outer[row:row + b.shape[0], col:col + b.shape[1]] = b
+                row, col = row + b.shape[0], col + b.shape[1]
+            self.outer = Linear(outer)
         self.out = Linear(t["o"])
         self.taps = torch.cat([t["q_conv"], t["k_conv"], t["v_conv"]], dim=0).contiguous()
         self.A_log, self.dt_bias, self.norm_weight = t["A_log"], t["dt_bias"], t["norm"]
@@ -116,14 +151,23 @@ class GatedDeltaRule(Mixer):
         """The heads' normed and gated read-outs [rows, heads * vdim] in the activation dtype; the
         request's state moves on by the step's rows."""
         proj = self.in_proj.forward(h, out_dtype=torch.float32)
-        both = self.outer.forward(self.low.forward(h), out_dtype=torch.float32)
-        a, gate = both[:, :self.heads * self.dim], both[:, self.heads * self.dim:]
+        both = self.outer.forward(self.low.forward(h), out_dtype=torch.float32) if self.outer is not None else None
+        per_head = self.decay == "head"
+        if per_head:
+            a = proj[:, self.a_col:self.a_col + self.heads]
+        else:
+            a = both[:, :self.heads * self.dim]
+        if self.gate == "silu":
+            gate = proj[:, self.gate_col:self.gate_col + self.heads * self.vdim]
+        else:
+            gate = both[:, both.shape[1] - self.heads * self.vdim:]
         records = ops.delta_prepare(proj, self.beta_col, a, self.taps, self._conv_state(cache), self.A_log, self.dt_bias,
                                     ctx.row_seg, ctx.seg_row0, ctx.seg_slot, ctx.num_segments, self.heads, self.kv_heads,
-                                    self.dim, self.vdim)
+                                    self.dim, self.vdim, decay_per_head=per_head)
         o = ops.gated_delta_rule(records, cache["state"].state, ctx.seg_row0, ctx.seg_slot, ctx.num_segments,
                                  self.heads, self.dim, self.vdim)
-        return ops.gated_head_norm(o, gate, self.norm_weight, self.heads, self.vdim, self.eps, self.dtype)
+        return ops.gated_head_norm(o, gate, self.norm_weight, self.heads, self.vdim, self.eps, self.dtype,
+                                   gate_silu=self.gate == "silu")
 
     def output(self, h, ctx, cache) -> torch.Tensor:
         return self.out.forward(self.heads_output(h, ctx, cache), out_dtype=torch.float32)

@@ -1,0 +1,126 @@
+"""Attention over a cached latent, without positions.
+
+The query passes a low-rank map with a norm in its middle: c_q = rms(W_dq h) * w_q, q = W_uq c_q
+(heads of ``head_dim`` channels). Keys and values of every head are linear maps of one latent per
+token, c = rms(W_dkv h) * w_kv (``kv_rank`` channels): k_i = W_uk,i c, v_i = W_uv,i c (values of
+``v_head_dim`` channels). Scores q_i . k_i * softmax_scale over every earlier token and the row itself,
+softmax in float32; the heads side by side are multiplied by sigmoid(W_g h) and pass W_o.
+
+Only c is cached, and the two maps move to the query's side of the products: q_i . (W_uk,i c) =
+(W_uk,i^T q_i) . c, and sum_j p_j (W_uv,i c_j) = W_uv,i (sum_j p_j c_j). The paged attention kernels then
+see ``num_heads`` query heads of ``kv_rank`` channels over ONE key/value head whose keys and values are
+both c (each in the layout its product reduces over), whatever the number of heads; the gate rides in
+the epilogue of the map back to the values' size. An RMS norm here is x / sqrt(mean(x^2) + eps).
+"""
+
+from __future__ import annotations
+
+from typing import Dict
+
+import torch
+
+from ..cache.needs import PagedKV
+from ..config.spec import ConfigError
+from ..kernels import ops
+from ..weights.loader import TensorDecl
+from .attention import GQAttention
+from .base import Mixer, register_mixer
+from .linear import Linear
+
+_DEFAULT_NAMES = {"dq": "dq", "dq_norm": "dq.norm", "uq": "uq", "dkv": "dkv", "dkv_norm": "dkv.norm", "uk": "uk", "uv": "uv",
+                  "g": "g", "o": "o"}
+
+
+@register_mixer("latent_attention")
+class LatentAttention(Mixer):
+    graph_safe = True
+    RUN_OF_KEYS = GQAttention.RUN_OF_KEYS
+
+    def __init__(self, spec):
+        super().__init__(spec)
+        self.hidden = int(spec["hidden_size"])
+        self.num_heads = int(spec["num_heads"])
+        self.head_dim = int(spec["head_dim"])
+        self.v_head_dim = int(spec.get("v_head_dim") or self.head_dim)
+        self.q_rank = int(spec["q_rank"])
+        self.kv_rank = int(spec["kv_rank"])
+        self.eps = float(spec["norm_eps"])
+        self.scale = float(spec.get("softmax_scale", self.head_dim ** -0.5))
+        self.gated = bool(spec.get("output_gate", True))
+        self.names = {**_DEFAULT_NAMES, **dict(spec.get("names", {}))}
+        if not 1 <= self.kv_rank <= ops.MAX_HEAD_DIM:
+            raise ConfigError(f"a latent of {self.kv_rank} channels exceeds the attention kernels' limit of {ops.MAX_HEAD_DIM}")
+        if min(self.num_heads, self.head_dim, self.v_head_dim, self.q_rank) < 1:
+            raise ConfigError("latent attention: every size must be positive")
+
+    def cache_need(self):
+        return PagedKV(1, self.kv_rank, None, None)
+
+    def _name(self, which: str) -> str:
+        return self.prefix + self.names[which]
+
+    def tensors(self) -> Dict[str, TensorDecl]:
+        D, H, d, dv, rq, rk = self.hidden, self.num_heads, self.head_dim, self.v_head_dim, self.q_rank, self.kv_rank
+        declared = {
+            self._name("dq"): TensorDecl((rq, D)), self._name("dq_norm"): TensorDecl((rq,), "vector", "norm"),
+            self._name("uq"): TensorDecl((H * d, rq)),
+            self._name("dkv"): TensorDecl((rk, D)), self._name("dkv_norm"): TensorDecl((rk,), "vector", "norm"),
+            self._name("uk"): TensorDecl((H * d, rk)), self._name("uv"): TensorDecl((H * dv, rk)),
+            self._name("o"): TensorDecl((D, H * dv)),
+        }
+        if self.gated:
+            declared[self._name("g")] = TensorDecl((H * dv, D))
+        return declared
+
+    def bind(self, tensors, dtype, device) -> None:
+        super().bind(tensors, dtype, device)
+        t = {which: tensors[self._name(which)] for which in self.names if self._name(which) in tensors}
+        H, d, dv, rk = self.num_heads, self.head_dim, self.v_head_dim, self.kv_rank
+        # what reads h: the query's inner map, and the latent's with the gate behind it in one operand
+        # (float32 sums out: the norms and the sigmoid read them as they are)
+        self.down_q = Linear(t["dq"])
+        self.down_kv = Linear(torch.cat([t["dkv"], t["g"]], dim=0) if self.gated else t["dkv"])
+        self.up_q = Linear(t["uq"])
+        # per head: the keys' map transposed (it is applied to the query), the values' map as it is
+        self.uk_t = t["uk"].reshape(H, d, rk).transpose(1, 2).contiguous()       # [H][rk][d]
+        self.uv = t["uv"].reshape(H, dv, rk).contiguous()                        # [H][dv][rk]
+        self.out = Linear(t["o"])
+        self.q_norm_weight, self.kv_norm_weight = t["dq_norm"], t["dkv_norm"]
+
+    # the matrix-core attention kernels need the step's query tiles, as grouped-query attention does
+    def _fast(self) -> bool:
+        return getattr(self, "dtype", None) == torch.bfloat16 and ops.attention_is_tiled(self.kv_rank)
+
+    def step_arrays_key(self):
+        return ("query_tiles", ops.QUERY_TILE, self.RUN_OF_KEYS) if self._fast() else None
+
+    step_arrays = GQAttention.step_arrays
+    refresh_step_arrays = GQAttention.refresh_step_arrays
+    _decode_work = GQAttention._decode_work
+
+    def mixing_flops(self, rows: int, keys_before: int = 0) -> int:
+        """Scores and weighted sums over the latent for rows that follow ``keys_before`` cached tokens,
+        and the two maps per head around them."""
+        pairs = rows * keys_before + rows * (rows + 1) // 2
+        return 4 * self.num_heads * self.kv_rank * pairs + 2 * rows * self.num_heads * self.kv_rank * (self.head_dim + self.v_head_dim)
+
+    def heads_output(self, h, ctx, cache) -> torch.Tensor:
+        """The gated heads [rows, heads * v_head_dim] in the activation dtype; the step's latents join the cache."""
+        down = self.down_kv.forward(h, out_dtype=torch.float32)
+        if cache.writes:
+            ops.latent_norm_write(down[:, :self.kv_rank], self.kv_norm_weight, self.eps, cache.k_pages, cache.v_pages,
+                                  cache.block_table, ctx.row_seg, ctx.row_pos)
+        c_q = ops.rmsnorm_rows(self.down_q.forward(h, out_dtype=torch.float32), self.q_norm_weight, self.eps, self.dtype)
+        q = self.up_q.forward(c_q)
+        q_latent = ops.head_linear(q, self.uk_t, self.dtype)                      # [rows, H * rk]
+        own = ctx.step_arrays(self) if self.step_arrays_key() is not None else {}
+        mixed = ops.attention(q_latent, self.num_heads, 1, self.kv_rank, cache.k_pages, cache.v_pages, cache.block_table, ctx,
+                              self.scale, 0, tile_seg=own.get("tile_seg"), tile_row0=own.get("tile_row0"),
+                              decode_work=own.get("decode_work"), v_dim=self.kv_rank)
+        return ops.head_linear(mixed, self.uv, self.dtype, gate=down[:, self.kv_rank:] if self.gated else None)
+
+    def output(self, h, ctx, cache) -> torch.Tensor:
+        return self.out.forward(self.heads_output(h, ctx, cache), out_dtype=torch.float32)
+
+    def forward(self, h, residual, ctx, cache):
+        return self.out.accumulate(self.heads_output(h, ctx, cache), residual, then=getattr(ctx, "upcoming_norm", None))

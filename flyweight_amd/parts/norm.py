@@ -1,5 +1,6 @@
 """RMS norm: y = x * rsqrt(mean(x^2) + eps) * w, sums in float32; the weight multiplies
-directly (native/include/flyweight_v2_qwen_kernels.hpp:425-447 with one_centered = 0)."""
+directly (native/include/flyweight_v2_qwen_kernels.hpp:425-447 with one_centered = 0).
+Layer norm with a weight and no bias: the row's mean is taken off first, y = (x - m) * rsqrt(mean((x - m)^2) + eps) * w."""
 
 from __future__ import annotations
 
@@ -21,6 +22,15 @@ class Prepared:
         self.norm, self.activations, self.squares = norm, activations, squares
 
 
+class NormedRows:
+    """Rows that the kernel which last changed the residual stream has already passed through ``norm``
+    (``activations``, in the activation dtype): whoever is about to apply that very norm to those
+    very rows takes them instead."""
+
+    def __init__(self, norm: Norm, activations: torch.Tensor):
+        self.norm, self.activations = norm, activations
+
+
 class LazyNorm:
     """A norm that has not run yet: the rows ``x`` (optionally gathered through ``row_index``)
     and the norm to apply. A product that can apply an RMS norm in its own kernel takes it as
@@ -33,8 +43,10 @@ class LazyNorm:
         # only what was made for this very norm and these rows counts
         ok = prepared is not None and prepared.norm is norm and row_index is None \
             and prepared.activations.shape == x.shape
-        self.prepared = prepared if ok else None
         self._tensor = None
+        if ok and isinstance(prepared, NormedRows):     # the norm has run already
+            self._tensor, ok = prepared.activations, False
+        self.prepared = prepared if ok else None
 
     @property
     def rows(self) -> int:
@@ -80,6 +92,39 @@ class RMSNorm(Norm):
     def rms_parameters(self):
         return self.weight, self.eps, self.one_centered
 
+    def row_norm(self):
+        """(weight, eps, centered) for a kernel that applies the norm beside other work on the row, or
+        None where the norm is not of that plain form."""
+        return None if self.one_centered else (self.weight, self.eps, False)
+
     def forward(self, x: torch.Tensor, ctx, row_index: Optional[torch.Tensor] = None) -> torch.Tensor:
         return ops.rmsnorm_rows(x, self.weight, self.eps, self.dtype, row_index=row_index,
                                 one_centered=self.one_centered)
+
+
+@register_norm("layernorm")
+class LayerNorm(Norm):
+    """(x - mean) / sqrt(variance + eps) * w, the variance the mean of the squared deviations; no bias."""
+    graph_safe = True
+
+    def __init__(self, spec):
+        super().__init__(spec)
+        self.size = int(spec["size"])
+        self.eps = float(spec["eps"])
+
+    @property
+    def tensor_name(self) -> str:
+        return self.spec.get("tensor") or self.prefix + "weight"
+
+    def tensors(self) -> Dict[str, TensorDecl]:
+        return {self.tensor_name: TensorDecl((self.size,), role="vector", init="norm")}
+
+    def bind(self, tensors, dtype, device) -> None:
+        super().bind(tensors, dtype, device)
+        self.weight = tensors[self.tensor_name]
+
+    def row_norm(self):
+        return self.weight, self.eps, True
+
+    def forward(self, x: torch.Tensor, ctx, row_index: Optional[torch.Tensor] = None) -> torch.Tensor:
+        return ops.layernorm_rows(x, self.weight, self.eps, self.dtype, row_index=row_index)

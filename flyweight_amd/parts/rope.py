@@ -1,6 +1,8 @@
 """Rotary position encoding, half-split pairing: channel i of a head pairs with channel
 i + rotary_dim/2, angle = position * theta^(-2i/rotary_dim); channels past ``rotary_dim``
-pass through (native/include/flyweight_v2_native_kernels.hpp:993-1050). The inverse
+pass through (native/include/flyweight_v2_native_kernels.hpp:993-1050). ``rotary_interleaved``
+pairs channel 2i with channel 2i + 1 instead, by the same angles (``interleaved`` tells the mixer's
+kernels which pairing the tables are for). The inverse
 frequencies are formed in float64 on the host; the per-step cos/sin tables are float32.
 ``rotary_dim = 0`` (or kind ``none``) means no position encoding at all. ``scaling_factor`` f
 (linear position scaling) divides every frequency by f: position p turns as p / f would."""
@@ -17,6 +19,7 @@ from .base import PositionEncoding, register_position_encoding
 @register_position_encoding("rotary_neox")
 class RotaryNeox(PositionEncoding):
     graph_safe = True
+    interleaved = False
 
     def __init__(self, spec):
         super().__init__(spec)
@@ -40,6 +43,13 @@ class RotaryNeox(PositionEncoding):
         if self.rotary_dim == 0:
             return None, None
         return ops.rope_table(ctx.encoding_pos, self._inv_freq)
+
+
+@register_position_encoding("rotary_interleaved")
+class RotaryInterleaved(RotaryNeox):
+    """The pair (u, v) = (channel 2i, channel 2i + 1) becomes (u cos a - v sin a, v cos a + u sin a),
+    a = position * theta^(-2i / rotary_dim)."""
+    interleaved = True
 
 
 @register_position_encoding("none")

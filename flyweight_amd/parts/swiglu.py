@@ -27,9 +27,11 @@ class SwiGLU(FeedForward):
         self.hidden = int(spec["hidden_size"])
         self.intermediate = int(spec["intermediate_size"])
         self.names = {**_DEFAULT_NAMES, **dict(spec.get("names", {}))}
+        # what follows a tensor's name in the checkpoint: ".weight" unless the layout has none
+        self.weight_suffix = spec.get("weight_suffix", ".weight")
 
     def _name(self, which: str) -> str:
-        return f"{self.prefix}{self.names[which]}.weight"
+        return f"{self.prefix}{self.names[which]}{self.weight_suffix}"
 
     def tensors(self) -> Dict[str, TensorDecl]:
         return {
@@ -49,3 +51,8 @@ class SwiGLU(FeedForward):
     def forward(self, h, residual, ctx):
         # the activation is formed from float32 sums and rounded once
         return self.down.accumulate(self.gate_up.swiglu(h), residual, then=getattr(ctx, "upcoming_norm", None))
+
+    def output(self, h, ctx) -> torch.Tensor:
+        """The feed-forward's output as float32 rows of its own (for arrangements that do something to
+        it before it joins the residual stream)."""
+        return self.down.forward(self.gate_up.swiglu(h), out_dtype=torch.float32)
