@@ -83,6 +83,37 @@ def koketar_configs(size: dict):
     return koketar, lfm2
 
 
+# Vavelorn (layers of chunked attention, attention over a cached latent and a gated delta rule in turn, a norm
+# before and behind every sublayer, a token input per layer) at two such sizes, beside the engine's closest
+# existing model: a Koketar of the same width, depth, feed-forward width and vocabulary (windowed attention
+# beside a gated delta rule in every layer, norms on the sublayers' outputs).
+VAVELORN_SIZES = {
+    "w1024": dict(width=1024, layers=6, vocab=32768, ff=4096, heads=8, kv_heads=2, dim=128, vdim=128, window=512, rot_dims=64,
+                  r_heads=8, r_kv_heads=4, r_dim=64, r_vdim=128, conv=4, rank=32, q_rank=384, kv_rank=256, side=32),
+    "w2048": dict(width=2048, layers=6, vocab=32768, ff=8192, heads=16, kv_heads=4, dim=128, vdim=128, window=1024, rot_dims=64,
+                  r_heads=16, r_kv_heads=8, r_dim=128, r_vdim=128, conv=4, rank=64, q_rank=768, kv_rank=256, side=64),
+}
+
+
+def vavelorn_configs(size: dict):
+    """(Vavelorn configuration, Koketar configuration of equal size)."""
+    from flyweight_amd.config import config_from_dict
+    mlp = {"kind": "dense", "ff": size["ff"]}
+    kinds = [
+        {"type": "attention", "mlp": mlp,
+         "mixer": {"heads": size["heads"], "kv_heads": size["kv_heads"], "dim": size["dim"], "vdim": size["vdim"], "scale": size["dim"] ** -0.5,
+                   "softcap": 50.0, "mask": {"size": size["window"]}, "rot": {"dims": size["rot_dims"], "base": 1000000.0}}},
+        {"type": "latent_attention", "mlp": mlp,
+         "mixer": {"heads": size["heads"], "dim": size["dim"], "vdim": size["vdim"], "q_rank": size["q_rank"], "kv_rank": size["kv_rank"],
+                   "scale": size["dim"] ** -0.5}},
+        {"type": "delta", "mlp": mlp,
+         "mixer": {"heads": size["r_heads"], "kv_heads": size["r_kv_heads"], "dim": size["r_dim"], "vdim": size["r_vdim"], "conv": size["conv"]}},
+    ]
+    vavelorn = config_from_dict({"architecture": "Vavelorn", "vocab": size["vocab"], "width": size["width"], "norm": {"eps": 1e-5},
+                                 "token_side": {"dim": size["side"]}, "layers": [kinds[i % 3] for i in range(size["layers"])]})
+    return vavelorn, koketar_configs(size)[0]
+
+
 def kernel_times(torch, run) -> dict:
     """Entry point of the kernel library -> microseconds of GPU time per call, over one call of ``run``
     (launched kernel by kernel, every call bracketed by two events)."""
@@ -97,16 +128,19 @@ def kernel_times(torch, run) -> dict:
                    "us": round(t["gpu_ms"] * 1e3, 1)} for name, t in report.items()}
 
 
-def koketar_run(torch, args) -> dict:
+def koketar_run(torch, args, families=("koketar", "lfm2"), sizes=None, configs_of=None, title="Koketar",
+                beside="Koketar beside LFM2 at equal width, depth, feed-forward width and vocabulary") -> dict:
     """Prefill (one step of 2,048 prompt tokens) and decode (batch 8 and 64 behind 2,048-token prompts) of
-    Koketar and of the LFM2 of equal size, tokens a second, with the time of every kernel of a prompt's step
-    and of a decode step at batch 8."""
+    a model family and of the closest existing one at equal size (Koketar and LFM2 unless told otherwise),
+    tokens a second, with the time of every kernel of a prompt's step and of a decode step at batch 8."""
     from flyweight_amd import Model, Runtime, StepEntry
     import numpy as np
+    sizes = KOKETAR_SIZES if sizes is None else sizes
+    configs_of = koketar_configs if configs_of is None else configs_of
     results = {}
     steps = min(args.steps, 64)
-    if args.only:       # one phase of Koketar at width 2,048 alone, no JSON (for profiling)
-        config = koketar_configs(KOKETAR_SIZES["w2048"])[0]
+    if args.only:       # one phase of the first family at width 2,048 alone, no JSON (for profiling)
+        config = configs_of(sizes["w2048"])[0]
         model = Model.random(config, seed=0, dtype="bfloat16")
         if args.only == "prefill":
             seconds, _ = prefill_run(torch, model, config, repeats=3)
@@ -115,8 +149,8 @@ def koketar_run(torch, args) -> dict:
             seconds, _, _ = decode_run(torch, model, config, args.batch, steps, min(args.warmup, 8))
             log(f"{args.batch * steps / seconds:.1f} tokens/s")
         return None
-    for size_name, size in KOKETAR_SIZES.items():
-        for family, config in zip(("koketar", "lfm2"), koketar_configs(size)):
+    for size_name, size in sizes.items():
+        for family, config in zip(families, configs_of(size)):
             log(f"{family} {size_name}: random bfloat16 weights")
             model = Model.random(config, seed=0, dtype="bfloat16")
             record = {}
@@ -146,12 +180,12 @@ def koketar_run(torch, args) -> dict:
             results[f"{family}_{size_name}"] = record
             del model, runtime
             torch.cuda.empty_cache()
-    headline = results["koketar_w2048"]
-    return {"metric": "decode tok/s @ batch 8 (Koketar, width 2,048, 4 layers, 2,048-token prompts)",
+    headline = results[f"{families[0]}_w2048"]
+    return {"metric": f"decode tok/s @ batch 8 ({title}, width 2,048, {sizes['w2048']['layers']} layers, 2,048-token prompts)",
             "value": headline["decode_b8_tokens_per_s"], "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": min(args.warmup, 8),
             "ms_per_step": headline["decode_b8_ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
             "dtype": "bf16", "data": "synthetic: seeded uniform token ids, random-init weights",
-            "config": {"model": "Koketar beside LFM2 at equal width, depth, feed-forward width and vocabulary", "sizes": KOKETAR_SIZES,
+            "config": {"model": beside, "sizes": sizes,
                        "prompt_len": PROMPT, "seq_len": CONTEXT, "parallelism": "single GPU"},
             "results": results}
 
@@ -452,9 +486,10 @@ def main() -> int:
     parser.add_argument("--only", choices=("decode", "prefill"), help="run one phase and print no JSON (for profiling)")
     parser.add_argument("--drawn", action="store_true", help="with --only decode: the requests draw their tokens "
                         "(temperature 0.8, top_k 40, top_p 0.95, min_p 0.05) instead of taking the most likely one")
-    parser.add_argument("--workload", choices=("headline",) + tuple(WORKLOADS) + ("koketar",), default="headline",
+    parser.add_argument("--workload", choices=("headline",) + tuple(WORKLOADS) + ("koketar", "vavelorn"), default="headline",
                         help="headline: the LFM2-1.2B decode and prefill figures; long-context, mixed: a whole serving run; "
-                             "koketar: prefill and decode of Koketar beside LFM2 at equal sizes, kernel by kernel")
+                             "koketar: prefill and decode of Koketar beside LFM2 at equal sizes, kernel by kernel; "
+                             "vavelorn: the same of Vavelorn beside Koketar")
     parser.add_argument("--requests", type=int, help="requests of a serving workload (default: as the workload names)")
     args = parser.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -468,8 +503,12 @@ def main() -> int:
     from flyweight_amd import Model
     from flyweight_amd.config import config_from_dict
 
-    if args.workload == "koketar":
-        record = koketar_run(torch, args)
+    if args.workload in ("koketar", "vavelorn"):
+        if args.workload == "vavelorn":
+            record = koketar_run(torch, args, families=("vavelorn", "koketar"), sizes=VAVELORN_SIZES, configs_of=vavelorn_configs,
+                                 title="Vavelorn", beside="Vavelorn beside Koketar at equal width, depth, feed-forward width and vocabulary")
+        else:
+            record = koketar_run(torch, args)
         if record is not None:
             print(json.dumps(record), flush=True)
         return 0

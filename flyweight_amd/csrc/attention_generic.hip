@@ -70,7 +70,8 @@ __global__ __launch_bounds__(64) void qk_norm_rope_kv_write_kernel(
             const float other = normed[interleaved ? d ^ 1 : (d < half ? d + half : d - half)];
             const float c = cos_table[(size_t)row * half + pair];
             const float s = sin_table[(size_t)row * half + pair];
-            value = is_first ? value * c - other * s : value * c + other * s;
+            // one rounding of other * s, then one fused step: the same in every kernel that rotates
+            value = fmaf(value, c, is_first ? -(other * s) : other * s);
         }
         store_from_float(dest, d, value);
     }
@@ -158,7 +159,7 @@ __global__ __launch_bounds__(64) void qk_norm_rope_kv_write_rows_kernel(
             value = value * inv * w;
         }
         const float other = __shfl(value, partner & 63, 64);
-        if (lane < rotary_dim) value = is_first ? value * c[i] - other * sn[i] : value * c[i] + other * sn[i];
+        if (lane < rotary_dim) value = fmaf(value, c[i], is_first ? -(other * sn[i]) : other * sn[i]);
         T* dest = is_query ? q_out + ((size_t)row_of[i] * num_heads + vec) * head_dim
                            : k_pages + (((size_t)page[i] * num_kv_heads + (vec - num_heads)) * ATTN_PAGE + slot) * head_dim;
         if (active) store_from_float(dest, lane, value);

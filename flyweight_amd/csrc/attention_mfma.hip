@@ -483,7 +483,7 @@ __device__ __forceinline__ void norm_rotate_vector(const float* __restrict__ sou
             const int pair = interleaved ? d >> 1 : (d < half ? d : d - half);
             const float other = scratch[interleaved ? d ^ 1 : (d < half ? d + half : d - half)];
             const float c = cos_row[pair], s = sin_row[pair];
-            value = is_first ? value * c - other * s : value * c + other * s;
+            value = fmaf(value, c, is_first ? -(other * s) : other * s);
         }
         store(d, value);
     }

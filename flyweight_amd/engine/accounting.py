@@ -20,6 +20,9 @@ def _walk(obj, seen: set) -> Iterator:
     if isinstance(obj, (torch.Tensor, Linear)):
         yield obj
         return
+    if hasattr(obj, "gathered_tensors"):        # tables a part reads by the row: not weights that a step streams
+        for table in obj.gathered_tensors():
+            seen.add(id(table))
     if isinstance(obj, dict):
         children = list(obj.values())
     elif isinstance(obj, (list, tuple)):
@@ -87,7 +90,9 @@ def attention_flops(model, rows: int, keys_before: int = 0) -> int:
             need = mixer.cache_need()
             if need is None or isinstance(need, dict) or not need.paged or not hasattr(mixer, "num_heads"):
                 continue
-            if need.window:     # visible keys of row r: min(keys_before + r + 1, window)
+            if getattr(mixer, "chunk", 0):      # a row sees the keys of its own chunk: its place in the chunk, and itself
+                pairs = sum((keys_before + row) % mixer.chunk + 1 for row in range(rows))
+            elif need.window:     # visible keys of row r: min(keys_before + r + 1, window)
                 full = max(0, min(rows, need.window - keys_before - 1))     # rows that still see fewer than a window
                 pairs = full * keys_before + full * (full + 1) // 2 + (rows - full) * need.window
             else:

@@ -55,6 +55,10 @@ class TokenInput(Part):
     def row_norm(self):
         return self.weight, self.eps, False
 
+    def gathered_tensors(self):
+        """What the part reads by the row (a step's accounting does not count it among the weights it streams)."""
+        return (self.table,)
+
     def output(self, x_rounded: torch.Tensor, ctx) -> torch.Tensor:
         """``x_rounded``: the residual rows in the activation dtype. Returns y, float32 [rows, hidden]."""
         z = self.gate.forward(x_rounded, out_dtype=torch.float32)

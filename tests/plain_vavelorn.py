@@ -68,6 +68,23 @@ def rotate_pairs(x: np.ndarray, positions: np.ndarray, dims: int, base: float) -
 
 
 # ----- mixer: chunked attention ---------------------------------------------------------------
+def chunked_heads(q: np.ndarray, k: np.ndarray, v: np.ndarray, scale: float, size: Optional[int], cap: Optional[float]) -> np.ndarray:
+    """q [T, H, d], k [T, G, d], v [T, G, dv] of one sequence from position 0 -> [T, H, dv]: row i sees
+    the keys j <= i of its own chunk (i // size == j // size; no size: all), scores capped softly."""
+    T, H = q.shape[:2]
+    G = k.shape[1]
+    out = np.zeros((T, H, v.shape[2]))
+    for head in range(H):
+        g = head // (H // G)
+        for i in range(T):
+            lo = 0 if not size else (i // size) * size
+            score = (k[lo:i + 1, g] @ q[i, head]) * scale
+            if cap:
+                score = cap * np.tanh(score / cap)
+            out[i, head] = softmax_rows(score) @ v[lo:i + 1, g]
+    return out
+
+
 def chunked_attention(h: np.ndarray, w: Dict[str, np.ndarray], p: dict) -> np.ndarray:
     T = h.shape[0]
     H, G, d, dv = p["heads"], p["kv_heads"], p["dim"], p["vdim"]
@@ -78,17 +95,7 @@ def chunked_attention(h: np.ndarray, w: Dict[str, np.ndarray], p: dict) -> np.nd
     rot = p.get("rot") or {"dims": 0, "base": 1.0}
     q = rotate_pairs(q, positions, rot["dims"], rot["base"])
     k = rotate_pairs(k, positions, rot["dims"], rot["base"])
-    size = (p.get("mask") or {}).get("size")
-    cap = p.get("softcap")
-    out = np.zeros((T, H, dv))
-    for head in range(H):
-        g = head // (H // G)
-        for i in range(T):
-            lo = 0 if not size else (i // size) * size
-            score = (k[lo:i + 1, g] @ q[i, head]) * p["scale"]
-            if cap:
-                score = cap * np.tanh(score / cap)
-            out[i, head] = softmax_rows(score) @ v[lo:i + 1, g]
+    out = chunked_heads(q, k, v, p["scale"], (p.get("mask") or {}).get("size"), p.get("softcap"))
     return out.reshape(T, H * dv) @ w["o"].T
 
 
@@ -243,3 +250,36 @@ def tensor_shapes(config: dict) -> Dict[str, tuple]:
         if side:
             shapes.update({base + "side.gate": (side["dim"], D), base + "side.proj": (D, side["dim"]), base + "side.norm": (D,)})
     return shapes
+
+
+def greedy(config: dict, weights: Dict[str, np.ndarray], prompt, new: int) -> List[int]:
+    """The most likely token, ``new`` times (ties to the lowest id); the whole sequence is run again for each."""
+    tokens, out = list(prompt), []
+    for _ in range(new):
+        token = int(np.argmax(forward(config, weights, tokens)[-1]))
+        out.append(token)
+        tokens.append(token)
+    return out
+
+
+def random_weights(config: dict, seed: int) -> Dict[str, np.ndarray]:
+    """Weights that make every part count: matrices 1 / sqrt(columns) wide, norm weights of visible
+    spread, taps, decays and write strengths of visible size."""
+    rng = np.random.default_rng(seed)
+    out = {}
+    for name, shape in tensor_shapes(config).items():
+        leaf = name.split(".")[-1]
+        if leaf in ("norm1", "norm2", "norm1b", "norm2b", "norm") or name == "final.norm":
+            value = rng.uniform(0.6, 1.4, shape)
+        elif leaf == "conv":
+            value = rng.normal(0.0, 0.5, shape)
+        elif leaf == "A_log":
+            value = rng.uniform(-3.0, 0.5, shape)
+        elif leaf == "dt_bias":
+            value = rng.uniform(-3.0, 0.0, shape)
+        elif name == "side.embed":
+            value = rng.normal(0.0, 1.0, shape)
+        else:
+            value = rng.normal(0.0, 1.0 / math.sqrt(shape[-1]), shape)
+        out[name] = value
+    return out
