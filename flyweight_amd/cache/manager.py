@@ -167,12 +167,12 @@ class CacheManager:
             self.group_pages = [int(num_pages)] * len(grouped)
             default_pages = int(num_pages)
         # what bounds one sequence: the smallest pool among the groups that keep every key
-        keeping_all = [pages for pages, (need, _) in zip(self.group_pages, grouped.values()) if not need.window]
+        keeping_all = [pages for pages, (need, _) in zip(self.group_pages, grouped.values()) if not need.retention()]
         self.num_pages = min(keeping_all) if keeping_all else (max(self.group_pages) if self.group_pages else default_pages)
         self.max_pages_per_request = max_pages_per_request or max(self.group_pages, default=default_pages)
         # the bookkeeping lives in the host library
         self._lib = host.library()
-        windows = (ctypes.c_int * max(len(grouped), 1))(*[int(need.window or 0) for need, _ in grouped.values()])
+        windows = (ctypes.c_int * max(len(grouped), 1))(*[int(need.retention()) for need, _ in grouped.values()])
         if grouped:
             pages = (ctypes.c_int * len(grouped))(*self.group_pages)
             self._native = self._lib.fwh_cache_create_sized(len(grouped), windows, pages, max_requests, page_size,

@@ -30,6 +30,8 @@ class CacheView:
 
 
 class CacheNeed:
+    # a paged need that gives pages back says so to the bookkeeping through ``retention()``
+    # (0: every key is kept; see ``PagedKV.retention``); as inherited: its window, or 0
     """Interface of a need. ``paged`` True: ``allocate(units, ...)`` is called with the number of
     pages (the pool's pages and one spare behind them) and ``group_key()`` / ``window`` sort the
     entry into a page group; entries with equal keys share one pool and one block table per
@@ -42,6 +44,9 @@ class CacheNeed:
 
     def group_key(self) -> Tuple:
         raise NotImplementedError
+
+    def retention(self) -> int:
+        return int(self.window or 0)
 
     def allocate(self, units: int, page_size: int, dtype: torch.dtype, device: torch.device) -> Any:
         """The storage of one cache entry: any object; it is handed back to ``initial`` and ``view``."""
@@ -71,7 +76,9 @@ class PagedKV(CacheNeed):
     """Keys and values that grow with the sequence. Layers whose needs are equal share
     a group: one page pool and one block table per request. ``window`` None keeps all
     keys; a number keeps only the last ``window`` of them, and pages the window has
-    passed are given back. K keeps a key's channels together ([page][kv_head][token][channel]:
+    passed are given back. ``chunk``: a row sees the keys of its own chunk of that many
+    positions only (chunks counted from position 0), and the pages before the chunk of the
+    sequence's next token are given back. K keeps a key's channels together ([page][kv_head][token][channel]:
     the order the scores reduce over), V a channel's tokens ([page][kv_head][channel][token]:
     the order the weighted sum reduces over)."""
 
@@ -79,12 +86,23 @@ class PagedKV(CacheNeed):
     head_dim: int
     window: Optional[int] = None
     v_head_dim: Optional[int] = None        # the size of a value where it is not the keys' (None: head_dim)
+    chunk: Optional[int] = None
     paged = True
 
     def group_key(self) -> Tuple:
-        if self.v_head_dim in (None, self.head_dim):
-            return ("kv", self.num_kv_heads, self.head_dim, self.window)
-        return ("kv", self.num_kv_heads, self.head_dim, self.window, self.v_head_dim)
+        key = ("kv", self.num_kv_heads, self.head_dim, self.window)
+        if self.v_head_dim not in (None, self.head_dim):
+            key += (self.v_head_dim,)
+        if self.chunk:
+            key += ("chunk", self.chunk)
+        return key
+
+    def retention(self) -> int:
+        """What the bookkeeping is told: 0 every key is kept, w > 0 the last w, -c < 0 the keys of the next
+        token's chunk of c positions (with both, the window, which keeps no fewer pages than needed)."""
+        if self.window:
+            return int(self.window)
+        return -int(self.chunk) if self.chunk else 0
 
     def allocate(self, units, page_size, dtype, device):
         return (torch.zeros((units, self.num_kv_heads, page_size, self.head_dim), dtype=dtype, device=device),

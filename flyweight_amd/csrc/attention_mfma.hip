@@ -424,6 +424,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((HD <= 64 &
 }
 
 // ---- decode ------------------------------------------------------------------------------------
+#define MERGE_PARTS 64               // parts of a row up to which the last workgroup keeps their weights in LDS (a context of 16,384 tokens at one run each)
 #define DECODE_WORKGROUPS 512        // two per compute unit: beyond, longer splits serve better than more of them
 // grid (rows, kv heads * head tiles, splits); four waves, each takes one page of the split's
 // SPLIT_PAGES, and their results are merged in LDS in the order of the keys. Columns are the
@@ -499,6 +500,7 @@ __global__ __launch_bounds__(64 * SPLIT_PAGES) __attribute__((amdgpu_waves_per_e
     __shared__ f32x4 shared_o[SPLIT_PAGES][HD / 16][64];
     __shared__ float shared_m[SPLIT_PAGES][16], shared_l[SPLIT_PAGES][16];
     __shared__ int ticket_shared;
+    __shared__ float merge_w[MERGE_PARTS][16], merge_l[MERGE_PARTS][16];
     __shared__ __attribute__((aligned(16))) uint16_t fused_q[FUSED ? 16 : 1][FUSED ? HD : 8];
     __shared__ float fused_scratch[FUSED ? SPLIT_PAGES : 1][FUSED ? HD : 1];
     const int row = blockIdx.x, split = blockIdx.z;
@@ -589,7 +591,7 @@ __global__ __launch_bounds__(64 * SPLIT_PAGES) __attribute__((amdgpu_waves_per_e
     // how many workgroups work on this row: those whose first page holds a visible key
     const int row_splits = (last_block - first / PAGE + 1 + pages_per_split - 1) / pages_per_split;
     const int stride = PART_STRIDE(v_dim);
-    if (wave == 0 && valid) {
+    if (valid) {        // every wave: the four share out the channel tiles, each storing a quarter of the workgroup's result
         float m = NEG_BIG;
 #pragma unroll
         for (int w = 0; w < SPLIT_PAGES; ++w) m = fmaxf(m, shared_m[w][col]);
@@ -602,8 +604,9 @@ __global__ __launch_bounds__(64 * SPLIT_PAGES) __attribute__((amdgpu_waves_per_e
         float* dest = partial + (((size_t)row * num_heads + head) * max_splits + split) * stride;
         uint16_t* final_dest = out + ((size_t)row * num_heads + head) * v_dim;
 #pragma unroll
-        for (int t = 0; t < HD / 16; ++t) {
-            if (t * 16 >= v_dim) break;
+        for (int tt = 0; tt < (HD / 16 + SPLIT_PAGES - 1) / SPLIT_PAGES; ++tt) {
+            const int t = tt * SPLIT_PAGES + wave;
+            if (t >= HD / 16 || t * 16 >= v_dim) break;
             f32x4 sum = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int w = 0; w < SPLIT_PAGES; ++w) sum += weight[w] * shared_o[w][t][lane];
@@ -619,7 +622,7 @@ __global__ __launch_bounds__(64 * SPLIT_PAGES) __attribute__((amdgpu_waves_per_e
                     __hip_atomic_store(dest + t * 16 + g * 4 + r, sum[r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
         }
-        if (g == 0 && row_splits > 1) {
+        if (wave == 0 && g == 0 && row_splits > 1) {
             __hip_atomic_store(dest + v_dim, m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             __hip_atomic_store(dest + v_dim + 1, total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
@@ -636,6 +639,78 @@ __global__ __launch_bounds__(64 * SPLIT_PAGES) __attribute__((amdgpu_waves_per_e
     if (ticket_shared != row_splits - 1) return;
     if (threadIdx.x == 0) __hip_atomic_store(ticket, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     const int columns = group - head_tile * 16 < 16 ? group - head_tile * 16 : 16;
+    if (row_splits <= MERGE_PARTS) {
+        // Up to MERGE_PARTS parts: a thread per head first forms the parts' weights (their maxima and sums asked
+        // for together, the weights kept in LDS), then every thread sums its outputs with many loads in flight:
+        // eight outputs by eight parts at a time. With many heads on one kv head (hundreds of outputs a thread)
+        // the walk below, one output after the other with each part's maximum and sum read again, took longer
+        // than the attention itself. The parts are added in the order of the keys.
+        if (threadIdx.x < columns) {
+            const float* source = partial + ((size_t)row * num_heads + kvh * group + head_tile * 16 + threadIdx.x) * max_splits * stride;
+            float m = NEG_BIG;
+            for (int sp0 = 0; sp0 < row_splits; sp0 += 8) {
+                float ms[8], ls[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    const int sp = sp0 + u < row_splits ? sp0 + u : row_splits - 1;
+                    ms[u] = __hip_atomic_load(source + (size_t)sp * stride + v_dim, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    ls[u] = __hip_atomic_load(source + (size_t)sp * stride + v_dim + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+#pragma unroll
+                for (int u = 0; u < 8; ++u)
+                    if (sp0 + u < row_splits) {
+                        merge_w[sp0 + u][threadIdx.x] = ms[u];
+                        merge_l[sp0 + u][threadIdx.x] = ls[u];
+                        m = fmaxf(m, ms[u]);
+                    }
+            }
+            float total = 0.0f;
+            for (int sp = 0; sp < row_splits; ++sp) {
+                const float weight = exp2f(merge_w[sp][threadIdx.x] - m);
+                total += weight * merge_l[sp][threadIdx.x];
+                merge_w[sp][threadIdx.x] = weight;
+            }
+            merge_l[0][threadIdx.x] = 1.0f / total;
+        }
+        __syncthreads();
+        const int items = columns * v_dim;
+        for (int item0 = threadIdx.x; item0 < items; item0 += 64 * SPLIT_PAGES * 8) {
+            float acc[8];
+            const float* source[8];
+            int column[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int item = item0 + 64 * SPLIT_PAGES * u < items ? item0 + 64 * SPLIT_PAGES * u : items - 1;
+                column[u] = item / v_dim;
+                source[u] = partial + ((size_t)row * num_heads + kvh * group + head_tile * 16 + column[u]) * max_splits * stride + item % v_dim;
+                acc[u] = 0.0f;
+            }
+            for (int sp0 = 0; sp0 < row_splits; sp0 += 8) {
+                float vs[8][8];
+#pragma unroll
+                for (int q = 0; q < 8; ++q) {
+                    const int sp = sp0 + q < row_splits ? sp0 + q : row_splits - 1;
+#pragma unroll
+                    for (int u = 0; u < 8; ++u)
+                        vs[u][q] = __hip_atomic_load(source[u] + (size_t)sp * stride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+#pragma unroll
+                for (int q = 0; q < 8; ++q)
+                    if (sp0 + q < row_splits) {
+#pragma unroll
+                        for (int u = 0; u < 8; ++u) acc[u] += merge_w[sp0 + q][column[u]] * vs[u][q];
+                    }
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int item = item0 + 64 * SPLIT_PAGES * u;
+                if (item < items)
+                    out[((size_t)row * num_heads + kvh * group + head_tile * 16 + column[u]) * v_dim + item % v_dim] =
+                        float_to_bf16_bits(acc[u] * merge_l[0][column[u]]);
+            }
+        }
+        return;
+    }
     for (int item = threadIdx.x; item < columns * v_dim; item += 64 * SPLIT_PAGES) {
         const int merged_head = kvh * group + head_tile * 16 + item / v_dim, d = item % v_dim;
         const float* source = partial + ((size_t)row * num_heads + merged_head) * max_splits * stride;

@@ -52,7 +52,9 @@ private:
 constexpr int NO_PAGE = -1;
 
 struct Group {
-    int window;                                             // 0: every key is kept
+    // Which keys a sequence still needs: 0: every key; w > 0: the last w (a sliding window); -c < 0: those of
+    // the chunk of c positions that the next token falls into (chunks counted from position 0).
+    int window;
     Pool pool;
     std::unordered_map<int64_t, std::vector<int>> tables;   // request -> page per block (NO_PAGE once given back)
     Group(int window_, int pages) : window(window_), pool(pages) {}
@@ -79,7 +81,7 @@ public:
             if (page_size <= 0 || count <= 0) throw std::invalid_argument("page size and page count must be positive");
             largest = count > largest ? count : largest;
             // what bounds a sequence: the smallest pool among the groups that keep every key
-            const bool keeps_all = g >= windows.size() || windows[g] <= 0;
+            const bool keeps_all = g >= windows.size() || windows[g] == 0;
             if (keeps_all && (num_pages_ == 0 || count < num_pages_)) num_pages_ = count;
             if (g < windows.size()) groups_.emplace_back(windows[g], count);
         }
@@ -98,10 +100,12 @@ public:
 
     int pages_for(int tokens) const { return (tokens + page_size_ - 1) / page_size_; }
 
-    // Blocks before this one hold only keys the window has passed once the sequence is
-    // `length` tokens long (the next query sits at position `length`).
+    // Blocks before this one hold only keys the window has passed (or that lie before the chunk
+    // of the next token) once the sequence is `length` tokens long (the next query sits at
+    // position `length`).
     int first_needed_block(const Group& group, int length) const {
-        if (group.window <= 0) return 0;
+        if (group.window == 0) return 0;
+        if (group.window < 0) return (length - length % -group.window) / page_size_;
         const int first_key = length - group.window + 1 > 0 ? length - group.window + 1 : 0;
         return first_key / page_size_;
     }

@@ -30,7 +30,8 @@ int fwh_pool_free_count(void* pool);
 int fwh_pool_peak(void* pool);                  // most ids out at any time
 int fwh_pool_is_held(void* pool, int id);
 
-// ---- the cache: page groups (window 0: every key is kept), block tables, slots --------------------
+// ---- the cache: page groups (window 0: every key is kept; w > 0: the last w keys; -c < 0: the keys of the
+// ---- chunk of c positions that the next token falls into), block tables, slots ------------------------
 void* fwh_cache_create(int num_groups, const int* windows, int num_pages, int max_requests, int page_size,
                        int max_pages_per_request);
 // the same with a pool size per group (a group that keeps a window needs fewer pages than one that keeps every key)

@@ -118,15 +118,98 @@ __global__ __launch_bounds__(256) void head_linear_kernel(const TI* __restrict__
     }
 }
 
+// The same on the matrix cores, bfloat16 in, float32 sums, bfloat16 out. A wave forms 16 rows by 16 NT outputs of
+// one head: per 32 values of k one operand of the rows and NT of the weights, each lane's eight values
+// one 16-byte load straight from memory (K and the rows' stride multiples of 8), no LDS: the weights of a head are
+// few and stay in the caches for the waves that share them. The product is taken transposed (weights as
+// the first operand), so that a lane ends with four neighbouring outputs of one row. WIDE: the workgroup's
+// four waves take four runs of outputs of the same 16 rows (a decode step's few rows); else four runs of
+// rows for the same outputs. Each output's sum runs over k in the same order whatever the rows beside it.
+typedef __attribute__((ext_vector_type(8))) __bf16 hl_bf16x8;
+typedef __attribute__((ext_vector_type(4))) float hl_f32x4;
+typedef __attribute__((ext_vector_type(4))) uint32_t hl_u32x4;
+template <int NT, bool WIDE>
+__global__ __launch_bounds__(256) void head_linear_mfma_kernel(const uint16_t* __restrict__ in, int in_stride, const uint16_t* __restrict__ w,
+                                                              const float* __restrict__ gate, int gate_stride, uint16_t* __restrict__ out,
+                                                              int rows, int heads, int N, int K) {
+    const int head = blockIdx.z;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, i16 = lane & 15, g = lane >> 4;
+    const int row0 = WIDE ? blockIdx.x * 16 : (blockIdx.x * 4 + wave) * 16;
+    const int col0 = WIDE ? (blockIdx.y * 4 + wave) * 16 * NT : blockIdx.y * 16 * NT;
+    if (row0 >= rows || col0 >= N) return;
+    const int my_row = row0 + i16 < rows ? row0 + i16 : rows - 1;           // rows past the end compute along and store nothing
+    const uint16_t* a_from = in + (size_t)my_row * in_stride + (size_t)head * K + g * 8;
+    const uint16_t* w_from[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+        const int n = col0 + t * 16 + i16 < N ? col0 + t * 16 + i16 : N - 1;
+        w_from[t] = w + ((size_t)head * N + n) * K + g * 8;
+    }
+    hl_f32x4 acc[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) acc[t] = hl_f32x4{0.f, 0.f, 0.f, 0.f};
+    const hl_u32x4 zero = {0u, 0u, 0u, 0u};
+    for (int k0 = 0; k0 < K; k0 += 32) {
+        const bool k_in = k0 + g * 8 < K;
+        const hl_u32x4 a_bits = k_in ? *reinterpret_cast<const hl_u32x4*>(a_from + k0) : zero;
+        hl_u32x4 w_bits[NT];
+#pragma unroll
+        for (int t = 0; t < NT; ++t) w_bits[t] = k_in ? *reinterpret_cast<const hl_u32x4*>(w_from[t] + k0) : zero;
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+            acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(hl_bf16x8, w_bits[t]), __builtin_bit_cast(hl_bf16x8, a_bits), acc[t], 0, 0, 0);
+    }
+    fw_mfma_drain();        // the last products have left the pipe before a branch leads to code that reads them
+    if (row0 + i16 >= rows) return;
+    const int row = row0 + i16;
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+        const int n0 = col0 + t * 16 + g * 4;           // this lane: outputs n0 .. n0 + 3 of its row
+        float value[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            value[r] = acc[t][r];
+            if (gate && n0 + r < N) value[r] *= 1.0f / (1.0f + expf(-gate[(size_t)row * gate_stride + (size_t)head * N + n0 + r]));
+        }
+        uint16_t* dest = out + (size_t)row * heads * N + (size_t)head * N + n0;
+        if (n0 + 3 < N && N % 4 == 0) {
+            typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+            *reinterpret_cast<u32x2*>(dest) = u32x2{(uint32_t)float_to_bf16_bits(value[0]) | ((uint32_t)float_to_bf16_bits(value[1]) << 16),
+                                                    (uint32_t)float_to_bf16_bits(value[2]) | ((uint32_t)float_to_bf16_bits(value[3]) << 16)};
+        } else {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                if (n0 + r < N) dest[r] = float_to_bf16_bits(value[r]);
+        }
+    }
+}
+
 extern "C" int fw_head_linear(const void* in, int in_dtype, int in_stride, const void* w, int w_dtype, const float* gate,
                               int gate_stride, void* out, int out_dtype, int rows, int heads, int N, int K, void* stream) {
     FW_REQUIRE(rows >= 0 && heads > 0 && heads <= 65535 && N > 0 && K > 0, "head_linear: bad sizes rows=%d heads=%d N=%d K=%d", rows, heads, N, K);
     FW_REQUIRE(in_stride >= heads * K, "head_linear: rows %d wide do not hold %d x %d", in_stride, heads, K);
     FW_REQUIRE(gate == nullptr || gate_stride >= heads * N, "head_linear: the gates' rows (%d wide) do not hold %d x %d", gate_stride, heads, N);
     if (rows == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    if (in_dtype == FW_BF16 && w_dtype == FW_BF16 && out_dtype == FW_BF16 && K % 8 == 0 && in_stride % 8 == 0 && (uintptr_t)in % 16 == 0 &&
+        (uintptr_t)w % 16 == 0 && (uintptr_t)out % 8 == 0) {
+        // few rows: a wave per 16 outputs, so that a small product still spreads over the chip; else 64 outputs a wave
+        if (rows <= 16) {
+            dim3 wide(1, (N + 63) / 64, heads);
+            FW_REQUIRE(wide.y <= 65535, "head_linear: too many columns (%d)", N);
+            head_linear_mfma_kernel<1, true><<<wide, 256, 0, s>>>((const uint16_t*)in, in_stride, (const uint16_t*)w, gate, gate_stride,
+                                                                  (uint16_t*)out, rows, heads, N, K);
+        } else {
+            dim3 tall((rows + 63) / 64, (N + 63) / 64, heads);
+            FW_REQUIRE(tall.y <= 65535, "head_linear: too many columns (%d)", N);
+            head_linear_mfma_kernel<4, false><<<tall, 256, 0, s>>>((const uint16_t*)in, in_stride, (const uint16_t*)w, gate, gate_stride,
+                                                                   (uint16_t*)out, rows, heads, N, K);
+        }
+        FW_LAUNCH_CHECK("head_linear");
+        return 0;
+    }
     dim3 grid((rows + HL_TILE - 1) / HL_TILE, (N + HL_TILE - 1) / HL_TILE, heads);
     FW_REQUIRE(grid.y <= 65535, "head_linear: too many columns (%d)", N);
-    hipStream_t s = (hipStream_t)stream;
 #define FW_HL_LAUNCH(TI, TW, TO)                                                                                          \
     head_linear_kernel<TI, TW, TO><<<grid, 256, 0, s>>>((const TI*)in, in_stride, (const TW*)w, gate, gate_stride, \
                                                         (TO*)out, rows, heads, N, K)

@@ -68,7 +68,7 @@ class GQAttention(Mixer):
 
     def cache_need(self):
         return PagedKV(self.num_kv_heads, self.head_dim, None if self.window is None else int(self.window),
-                       None if self.v_head_dim == self.head_dim else self.v_head_dim)
+                       None if self.v_head_dim == self.head_dim else self.v_head_dim, self.chunk or None)
 
     def _name(self, which: str, leaf: str = "weight") -> str:
         if leaf == "weight":

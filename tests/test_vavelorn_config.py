@@ -63,7 +63,15 @@ def test_cache_entries(tmp_path):
     cache.admit("a")
     cache.reserve("a", 300)
     cache.commit("a", 300)
-    assert all(g.pool.in_use == 5 for g in cache.groups)
+    # the chunked group (chunks of 40) keeps the pages from the chunk of the next token on: position 300 lies in
+    # the chunk from 280, which begins in the fifth page; the groups that keep every key hold all five
+    held = {g.need.chunk: g.pool.in_use for g in cache.groups}
+    assert held == {40: 1, None: 5} and cache.groups[0].tables["a"][:4] == [-1, -1, -1, -1]
+    cache.reserve("a", 321)
+    cache.commit("a", 319)              # still in the chunk from 280: nothing more goes back
+    assert cache.groups[0].pool.in_use == 2
+    cache.commit("a", 320)              # the next token begins the chunk from 320, which lies in the sixth page
+    assert cache.groups[0].pool.in_use == 1 and cache.groups[0].tables["a"][4] == -1
     cache.release("a")
     cache.check_invariants()
     assert all(g.pool.in_use == 0 for g in cache.groups)
