@@ -19,7 +19,7 @@ from . import build as _build
 F32, BF16 = 0, 1
 PAGE_SIZE = 64          # tokens per cache page: the width of a wavefront
 MAX_HEAD_DIM = 256
-ABI_VERSION = 13
+ABI_VERSION = 14
 
 _lib = None
 

@@ -167,18 +167,22 @@ class SandwichNormResidualBlock(Block):
         position = getattr(self.mixer, "position", None)
         return all(part.graph_safe for part in self.parts()) and (position is None or position.graph_safe)
 
-    def _join(self, x, rows, norm, reader, dtype):
-        """x += norm(rows); returns what ``reader`` sees of the new x: a norm's output (``reader`` a norm),
-        x rounded (``reader`` "rounded"), or None (``reader`` None)."""
-        weight, eps, centered = norm.row_norm()
+    @staticmethod
+    def _reader(reader, dtype) -> dict:
+        """What a kernel that sums into x is told about the next reader of x: a norm (its output), "rounded"
+        (x in the activation dtype) or None."""
         if reader is None:
-            ops.norm_add_norm_(x, rows, weight, centered, eps)
-            return None
+            return {}
         if reader == "rounded":
-            return ops.norm_add_norm_(x, rows, weight, centered, eps, next_kind=ops.NEXT_ROUNDED, next_dtype=dtype)
+            return {"next_kind": ops.NEXT_ROUNDED, "next_dtype": dtype}
         next_weight, next_eps, next_centered = reader.row_norm()
-        return ops.norm_add_norm_(x, rows, weight, centered, eps, next_kind=ops.NEXT_CENTERED if next_centered else ops.NEXT_RMS,
-                                  next_weight=next_weight, next_eps=next_eps, next_dtype=dtype)
+        return {"next_kind": ops.NEXT_CENTERED if next_centered else ops.NEXT_RMS, "next_weight": next_weight, "next_eps": next_eps,
+                "next_dtype": dtype}
+
+    def _join(self, x, rows, norm, reader, dtype):
+        """x += norm(rows); returns what ``reader`` sees of the new x (None for no reader)."""
+        weight, eps, centered = norm.row_norm()
+        return ops.norm_add_norm_(x, rows, weight, centered, eps, **self._reader(reader, dtype))
 
     def forward(self, x, ctx, cache, prepared=None, norm_after=None):
         """``x`` [rows, hidden] float32 is updated in place."""
@@ -187,7 +191,7 @@ class SandwichNormResidualBlock(Block):
         after = norm_after if hasattr(norm_after, "row_norm") and norm_after.row_norm() is not None else None
         h = LazyNorm(self.mixer_norm, x, ctx, prepared=prepared).tensor()
         last = self.ffn is None and self.token_input is None
-        reader = after if last else (self.ffn_norm if self.ffn is not None else "rounded")
+        reader = after if last else (self.ffn_norm if self.ffn is not None else "rounded")     # the token input's product reads x rounded
         h = self._join(x, self.mixer.output(h, ctx, cache), self.mixer_post_norm, reader, dtype)
         if self.ffn is not None:
             reader = after if self.token_input is None else "rounded"

@@ -20,12 +20,13 @@ from typing import Dict
 import torch
 
 from ..cache.needs import PagedKV
-from ..config.spec import ConfigError
+from ..config.spec import ConfigError, PartSpec
 from ..kernels import ops
 from ..weights.loader import TensorDecl
 from .attention import GQAttention
-from .base import Mixer, register_mixer
+from .base import Mixer, build_part, register_mixer
 from .linear import Linear
+from .norm import LazyNorm
 
 _DEFAULT_NAMES = {"dq": "dq", "dq_norm": "dq.norm", "uq": "uq", "dkv": "dkv", "dkv_norm": "dkv.norm", "uk": "uk", "uv": "uv",
                   "g": "g", "o": "o"}
@@ -48,6 +49,8 @@ class LatentAttention(Mixer):
         self.scale = float(spec.get("softmax_scale", self.head_dim ** -0.5))
         self.gated = bool(spec.get("output_gate", True))
         self.names = {**_DEFAULT_NAMES, **dict(spec.get("names", {}))}
+        # the norm in the middle of the query's map is a norm part: the product behind it may take it into its own kernel
+        self.q_norm = build_part("norm", PartSpec("rmsnorm", {"size": self.q_rank, "eps": self.eps, "tensor": self._name("dq_norm")}))
         if not 1 <= self.kv_rank <= ops.MAX_HEAD_DIM:
             raise ConfigError(f"a latent of {self.kv_rank} channels exceeds the attention kernels' limit of {ops.MAX_HEAD_DIM}")
         if min(self.num_heads, self.head_dim, self.v_head_dim, self.q_rank) < 1:
@@ -62,7 +65,7 @@ class LatentAttention(Mixer):
     def tensors(self) -> Dict[str, TensorDecl]:
         D, H, d, dv, rq, rk = self.hidden, self.num_heads, self.head_dim, self.v_head_dim, self.q_rank, self.kv_rank
         declared = {
-            self._name("dq"): TensorDecl((rq, D)), self._name("dq_norm"): TensorDecl((rq,), "vector", "norm"),
+            self._name("dq"): TensorDecl((rq, D)), **self.q_norm.tensors(),
             self._name("uq"): TensorDecl((H * d, rq)),
             self._name("dkv"): TensorDecl((rk, D)), self._name("dkv_norm"): TensorDecl((rk,), "vector", "norm"),
             self._name("uk"): TensorDecl((H * d, rk)), self._name("uv"): TensorDecl((H * dv, rk)),
@@ -74,6 +77,7 @@ class LatentAttention(Mixer):
 
     def bind(self, tensors, dtype, device) -> None:
         super().bind(tensors, dtype, device)
+        self.q_norm.bind(tensors, dtype, device)
         t = {which: tensors[self._name(which)] for which in self.names if self._name(which) in tensors}
         H, d, dv, rk = self.num_heads, self.head_dim, self.v_head_dim, self.kv_rank
         # what reads h: the query's inner map, and the latent's with the gate behind it in one operand
@@ -85,7 +89,7 @@ class LatentAttention(Mixer):
         self.uk_t = t["uk"].reshape(H, d, rk).transpose(1, 2).contiguous()       # [H][rk][d]
         self.uv = t["uv"].reshape(H, dv, rk).contiguous()                        # [H][dv][rk]
         self.out = Linear(t["o"])
-        self.q_norm_weight, self.kv_norm_weight = t["dq_norm"], t["dkv_norm"]
+        self.kv_norm_weight = t["dkv_norm"]
 
     # the matrix-core attention kernels need the step's query tiles, as grouped-query attention does
     def _fast(self) -> bool:
@@ -110,8 +114,8 @@ class LatentAttention(Mixer):
         if cache.writes:
             ops.latent_norm_write(down[:, :self.kv_rank], self.kv_norm_weight, self.eps, cache.k_pages, cache.v_pages,
                                   cache.block_table, ctx.row_seg, ctx.row_pos)
-        c_q = ops.rmsnorm_rows(self.down_q.forward(h, out_dtype=torch.float32), self.q_norm_weight, self.eps, self.dtype)
-        q = self.up_q.forward(c_q)
+        # (for a few rows of a bfloat16 model the norm runs inside the product that reads it)
+        q = self.up_q.forward(LazyNorm(self.q_norm, self.down_q.forward(h, out_dtype=torch.float32), ctx))
         q_latent = ops.head_linear(q, self.uk_t, self.dtype)                      # [rows, H * rk]
         own = ctx.step_arrays(self) if self.step_arrays_key() is not None else {}
         mixed = ops.attention(q_latent, self.num_heads, 1, self.kv_rank, cache.k_pages, cache.v_pages, cache.block_table, ctx,
