@@ -162,6 +162,52 @@ def test_each_mixer_alone(models, name, variant, dtype):
     assert_close(feed(stepper, "c", tokens, [5, 2, 70, 1, 1]), loaded.expected(tokens), dtype, f"{name} {variant} cut")
 
 
+def random_config(seed):
+    """Two to six layers of any mixer in any order, every size drawn: heads and groups of 1..4, head sizes on
+    and off the matrix cores' steps of 16, chunks of 1 token to longer than the prompt or none, rotation of
+    none to all channels, latents of 8..256 channels, one to five taps, feed-forward widths that are no
+    multiple of eight or none, widths of 40..320, with and without a token input."""
+    from vavelorn_common import attention, delta, latent, layer
+    rng = np.random.default_rng(seed)
+    pick = lambda *xs: xs[int(rng.integers(len(xs)))]
+    layers = []
+    for _ in range(int(rng.integers(2, 7))):
+        kind = pick("attention", "latent_attention", "delta")
+        if kind == "attention":
+            kv, dim = int(pick(1, 2, 3, 4)), int(pick(16, 20, 32, 48, 64, 96, 128))
+            mixer = attention(kv * int(pick(1, 2, 3, 4)), kv, dim, int(pick(12, 16, 32, 64, 80, 128)), pick(None, 1, 7, 50, 64, 100, 128, 1000),
+                              int(pick(0, 2, 8, dim // 4 * 2, dim)), float(pick(100.0, 10000.0, 1e6)), float(pick(dim ** -0.5, 0.1, 0.3)),
+                              pick(None, 5.0, 30.0, 50.0))
+        elif kind == "latent_attention":
+            dim = int(pick(8, 16, 24, 64, 96))
+            mixer = latent(int(pick(1, 2, 3, 4, 8)), dim, int(pick(8, 20, 32, 80, 128)), int(pick(4, 24, 56, 64, 128)),
+                           int(pick(8, 36, 64, 96, 128, 200, 256)), float(pick(dim ** -0.5, 0.1, 0.25)))
+        else:
+            kv = int(pick(1, 2, 3))
+            mixer = delta(kv * int(pick(1, 2, 4)), kv, int(pick(4, 16, 24, 64, 128)), int(pick(4, 16, 40, 64, 128)), int(pick(1, 2, 3, 4, 5)))
+        layers.append(layer(mixer, pick(None, 70, 128, 256, 300)))
+    config = {"architecture": "Vavelorn", "vocab": int(pick(97, 300, 512, 1000)), "width": int(pick(40, 64, 96, 100, 128, 160, 192, 256, 320)),
+              "norm": {"eps": float(pick(1e-5, 1e-6))}, "layers": layers}
+    side = pick(None, 6, 8, 24, 40)
+    if side:
+        config["token_side"] = {"dim": int(side)}
+    return config
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_random_configurations(seed, tmp_path):
+    """Whatever config.json gives is read from there: ten drawn models, whole, token by token, in odd portions and
+    with a decoded tail, in both dtypes, against the plain model."""
+    config = random_config(seed)
+    tokens = random_tokens(config["vocab"], 150, seed=seed)
+    for dtype in DTYPES:
+        loaded = Loaded(str(tmp_path / dtype), config, dtype, seed=seed)
+        for cuts in ([150], [1], [3, 2, 64, 5, 2, 33, 65, 9], [130] + [1] * 20):
+            stepper = loaded.stepper(num_pages=4, max_requests=2)
+            stepper.admit("a")
+            assert_close(feed(stepper, "a", tokens, cuts), loaded.expected(tokens), dtype, f"drawn model {seed} cut {cuts[:3]}")
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name", ["X", "Y", "Z"])
 def test_mixed_batches_on_few_pages_and_slots(models, name, dtype):

@@ -127,7 +127,7 @@ def sharp_inputs(T, H, G, d, dv, sharp_keys, rng, strength=4.5):
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("chunk,rot_dims,d,dv,cap", [(64, 0, 32, 32, None), (65, 16, 32, 48, 30.0), (63, 32, 32, 16, 4.0),
-                                                      (120, 24, 96, 96, 50.0), (1, 8, 16, 16, None), (None, 64, 64, 128, 8.0),
+                                                      (112, 20, 80, 96, 40.0), (1, 8, 16, 16, None), (None, 64, 64, 128, 8.0),
                                                       (40, 4, 20, 12, 5.0)])
 def test_chunked_attention_with_a_sharp_key_at_every_edge(dtype, chunk, rot_dims, d, dv, cap):
     """Keys at the first and last place of every chunk are sharp: rows see the sharp first key of their own
@@ -174,7 +174,7 @@ def test_chunked_attention_with_a_sharp_key_at_every_edge(dtype, chunk, rot_dims
     assert_close(got.float().cpu().numpy(), want[rows], dtype, f"single rows, chunk {chunk}", scale=1.0)
 
 
-@pytest.mark.parametrize("chunk,rot_dims,d,dv,cap", [(65, 16, 32, 48, 30.0), (120, 24, 96, 96, 50.0), (None, 64, 64, 128, 8.0)])
+@pytest.mark.parametrize("chunk,rot_dims,d,dv,cap", [(65, 16, 32, 48, 30.0), (112, 20, 80, 96, 40.0), (None, 64, 64, 128, 8.0)])
 def test_fused_decode_attention(chunk, rot_dims, d, dv, cap):
     """Rotation, cache write and attention of a single-token step in one kernel: the rows after a prompt,
     one by one, against the plain functions; what it stores serves the rows behind it."""
