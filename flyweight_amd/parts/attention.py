@@ -28,8 +28,49 @@ from .linear import Linear
 _DEFAULT_NAMES = {"q": "q_proj", "k": "k_proj", "v": "v_proj", "o": "o_proj", "q_norm": "q_norm", "k_norm": "k_norm"}
 
 
+class QueryTileArrays:
+    """What a mixer that runs the matrix-core attention kernels over the paged cache asks of a step's upload
+    (``Part.step_arrays``). The prompt kernel works on tiles of up to 64 rows of one segment: which tiles
+    there are, and in which order workgroups take them. The split-key decode kernel shares a step's work out
+    over the chip by the number of runs of keys (four pages each) that all the rows it serves see together: a
+    long row among short ones gets more workgroups, and a recorded step adapts as its requests grow. The
+    mixer says through ``uses_query_tiles()`` whether its sizes and dtype take those kernels."""
+
+    RUN_OF_KEYS = ops.DECODE_SPLIT_PAGES * ops.PAGE_SIZE
+
+    def uses_query_tiles(self) -> bool:
+        raise NotImplementedError
+
+    def step_arrays_key(self):
+        return ("query_tiles", ops.QUERY_TILE, self.RUN_OF_KEYS) if self.uses_query_tiles() else None
+
+    def _decode_work(self, batch) -> int:
+        single = batch.num_rows if batch.all_decode else batch.decode_prefix    # the rows that go to the decode kernel
+        positions = np.asarray(batch.host_row_pos[:single], dtype=np.int64)
+        return int(np.sum((positions + self.RUN_OF_KEYS) // self.RUN_OF_KEYS))
+
+    def step_arrays(self, batch):
+        seg_row0 = batch.host_seg_row0
+        tile_seg, tile_row0 = ops.query_tiles(seg_row0)
+        # Workgroups start in the order of the tiles: those that see the most keys go first, the short
+        # ones fill in behind. The tiles of the leading single rows stay in front (they go to the
+        # decode kernel and their tiles are skipped).
+        if len(tile_seg) - batch.decode_prefix > 1 and not batch.all_decode:
+            tile_seg, tile_row0 = np.asarray(tile_seg, dtype=np.int32), np.asarray(tile_row0, dtype=np.int32)
+            tile_end = np.minimum(tile_row0 + ops.QUERY_TILE, np.asarray(seg_row0, dtype=np.int32)[tile_seg + 1])
+            keys_seen = batch.host_row_pos[tile_end - 1].astype(np.int64)
+            keys_seen[:batch.decode_prefix] = np.iinfo(np.int64).max
+            order = np.argsort(-keys_seen, kind="stable")
+            tile_seg, tile_row0 = tile_seg[order], tile_row0[order]
+        return {"tile_seg": np.asarray(tile_seg, dtype=np.int32), "tile_row0": np.asarray(tile_row0, dtype=np.int32),
+                "decode_work": np.asarray([self._decode_work(batch)], dtype=np.int32)}
+
+    def refresh_step_arrays(self, batch, arrays) -> None:
+        arrays["decode_work"][0] = self._decode_work(batch)     # the tiles of single rows never change
+
+
 @register_mixer("gqa_attention")
-class GQAttention(Mixer):
+class GQAttention(QueryTileArrays, Mixer):
     graph_safe = True
     accepts_lazy_norm = True
     # Up to this many rows a decode step forms queries and keys inside the attention kernel (at 8 rows
@@ -106,41 +147,9 @@ class GQAttention(Mixer):
         self.q_norm_weight = tensors[self._name("q_norm")] if self.qk_norm else None
         self.k_norm_weight = tensors[self._name("k_norm")] if self.qk_norm else None
 
-    # The kernels on the matrix cores need index arrays of this part's own. The prompt kernel works
-    # on tiles of up to 64 rows of one segment: which tiles there are, and in which order workgroups
-    # take them. The split-key decode kernel shares a step's work out over the chip by the number of
-    # runs of keys (four pages each) that all the rows it serves see together: a long row among
-    # short ones gets more workgroups, and a recorded step adapts as its requests grow.
-    RUN_OF_KEYS = ops.DECODE_SPLIT_PAGES * ops.PAGE_SIZE
-
-    def step_arrays_key(self):
-        fast = getattr(self, "dtype", None) == torch.bfloat16 and ops.attention_is_tiled(self.head_dim) \
+    def uses_query_tiles(self) -> bool:
+        return getattr(self, "dtype", None) == torch.bfloat16 and ops.attention_is_tiled(self.head_dim) \
             and ops.attention_is_tiled(self.v_head_dim)
-        return ("query_tiles", ops.QUERY_TILE, self.RUN_OF_KEYS) if fast else None
-
-    def _decode_work(self, batch) -> int:
-        single = batch.num_rows if batch.all_decode else batch.decode_prefix    # the rows that go to the decode kernel
-        positions = np.asarray(batch.host_row_pos[:single], dtype=np.int64)
-        return int(np.sum((positions + self.RUN_OF_KEYS) // self.RUN_OF_KEYS))
-
-    def step_arrays(self, batch):
-        seg_row0 = batch.host_seg_row0
-        tile_seg, tile_row0 = ops.query_tiles(seg_row0)
-        # Workgroups start in the order of the tiles: those that see the most keys go first, the short
-        # ones fill in behind. The tiles of the leading single rows stay in front (they go to the
-        # decode kernel and their tiles are skipped).
-        if len(tile_seg) - batch.decode_prefix > 1 and not batch.all_decode:
-            tile_seg, tile_row0 = np.asarray(tile_seg, dtype=np.int32), np.asarray(tile_row0, dtype=np.int32)
-            tile_end = np.minimum(tile_row0 + ops.QUERY_TILE, np.asarray(seg_row0, dtype=np.int32)[tile_seg + 1])
-            keys_seen = batch.host_row_pos[tile_end - 1].astype(np.int64)
-            keys_seen[:batch.decode_prefix] = np.iinfo(np.int64).max
-            order = np.argsort(-keys_seen, kind="stable")
-            tile_seg, tile_row0 = tile_seg[order], tile_row0[order]
-        return {"tile_seg": np.asarray(tile_seg, dtype=np.int32), "tile_row0": np.asarray(tile_row0, dtype=np.int32),
-                "decode_work": np.asarray([self._decode_work(batch)], dtype=np.int32)}
-
-    def refresh_step_arrays(self, batch, arrays) -> None:
-        arrays["decode_work"][0] = self._decode_work(batch)     # the tiles of single rows never change
 
     def attend(self, h, ctx, cache) -> torch.Tensor:
         """The heads' outputs [rows, heads * v_head_dim] in the activation dtype, the step's keys and

@@ -23,7 +23,7 @@ from ..cache.needs import PagedKV
 from ..config.spec import ConfigError, PartSpec
 from ..kernels import ops
 from ..weights.loader import TensorDecl
-from .attention import GQAttention
+from .attention import QueryTileArrays
 from .base import Mixer, build_part, register_mixer
 from .linear import Linear
 from .norm import LazyNorm
@@ -33,9 +33,8 @@ _DEFAULT_NAMES = {"dq": "dq", "dq_norm": "dq.norm", "uq": "uq", "dkv": "dkv", "d
 
 
 @register_mixer("latent_attention")
-class LatentAttention(Mixer):
+class LatentAttention(QueryTileArrays, Mixer):
     graph_safe = True
-    RUN_OF_KEYS = GQAttention.RUN_OF_KEYS
 
     def __init__(self, spec):
         super().__init__(spec)
@@ -91,16 +90,8 @@ class LatentAttention(Mixer):
         self.out = Linear(t["o"])
         self.kv_norm_weight = t["dkv_norm"]
 
-    # the matrix-core attention kernels need the step's query tiles, as grouped-query attention does
-    def _fast(self) -> bool:
+    def uses_query_tiles(self) -> bool:
         return getattr(self, "dtype", None) == torch.bfloat16 and ops.attention_is_tiled(self.kv_rank)
-
-    def step_arrays_key(self):
-        return ("query_tiles", ops.QUERY_TILE, self.RUN_OF_KEYS) if self._fast() else None
-
-    step_arrays = GQAttention.step_arrays
-    refresh_step_arrays = GQAttention.refresh_step_arrays
-    _decode_work = GQAttention._decode_work
 
     def mixing_flops(self, rows: int, keys_before: int = 0) -> int:
         """Scores and weighted sums over the latent for rows that follow ``keys_before`` cached tokens,
