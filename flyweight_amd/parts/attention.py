@@ -98,8 +98,8 @@ class GQAttention(QueryTileArrays, Mixer):
         self.position = build_part("position", spec["position"])
         if self.num_heads % self.num_kv_heads:
             raise ConfigError(f"{self.num_heads} heads are not a multiple of {self.num_kv_heads} kv heads")
-        if max(self.head_dim, self.v_head_dim) > ops.MAX_HEAD_DIM:
-            raise ConfigError(f"head_dim {self.head_dim} / value size {self.v_head_dim} exceeds the kernels' limit of {ops.MAX_HEAD_DIM}")
+        if max(self.head_dim, self.v_head_dim) > ops.MAX_PLAIN_HEAD_DIM:
+            raise ConfigError(f"head_dim {self.head_dim} / value size {self.v_head_dim} exceeds the kernels' limit of {ops.MAX_PLAIN_HEAD_DIM}")
         if self.bias and self.weight_suffix != ".weight":
             raise ConfigError("biases need the '.weight' / '.bias' tensor names")
         if self.window is not None and int(self.window) <= 0:

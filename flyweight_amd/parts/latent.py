@@ -50,8 +50,8 @@ class LatentAttention(QueryTileArrays, Mixer):
         self.names = {**_DEFAULT_NAMES, **dict(spec.get("names", {}))}
         # the norm in the middle of the query's map is a norm part: the product behind it may take it into its own kernel
         self.q_norm = build_part("norm", PartSpec("rmsnorm", {"size": self.q_rank, "eps": self.eps, "tensor": self._name("dq_norm")}))
-        if not 1 <= self.kv_rank <= ops.MAX_HEAD_DIM:
-            raise ConfigError(f"a latent of {self.kv_rank} channels exceeds the attention kernels' limit of {ops.MAX_HEAD_DIM}")
+        if not 1 <= self.kv_rank <= ops.MAX_PLAIN_HEAD_DIM:     # (beyond the matrix-core kernels' 256 channels the plain kernel serves)
+            raise ConfigError(f"a latent of {self.kv_rank} channels exceeds the attention kernels' limit of {ops.MAX_PLAIN_HEAD_DIM}")
         if min(self.num_heads, self.head_dim, self.v_head_dim, self.q_rank) < 1:
             raise ConfigError("latent attention: every size must be positive")
 

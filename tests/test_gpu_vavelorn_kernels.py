@@ -205,7 +205,7 @@ def test_fused_decode_attention(chunk, rot_dims, d, dv, cap):
 
 # ----- the latent ---------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("rank", [8, 40, 64, 128, 256])
+@pytest.mark.parametrize("rank", [8, 40, 64, 128, 256, 320])
 def test_latent_norm_and_store(dtype, rank):
     from flyweight_amd.kernels import ops
     rng = np.random.default_rng(rank)

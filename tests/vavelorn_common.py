@@ -64,7 +64,7 @@ CONFIG_Y = {
 
 # Z: the corners. A chunk of one token (a row sees itself alone) and one longer than any prompt here; no
 # rotation at all; one tap (no convolution memory) and six; heads of 4 and 8 channels; one head on one key
-# head and six on three; a latent of 8 channels and one query rank of 4; a feed-forward width that is no
+# head and six on three; a latent of 8 channels with a query rank of 4, and one of 320 channels; a feed-forward width that is no
 # multiple of eight; layers without feed-forward; no token input at all.
 CONFIG_Z = {
     "architecture": "Vavelorn", "vocab": 97, "width": 40, "norm": {"eps": 1e-5},
@@ -74,6 +74,7 @@ CONFIG_Z = {
         layer(latent(1, 8, 4, 4, 8, 0.5), None),
         layer(attention(6, 3, 24, 8, 500, 24, 10000.0, 0.25, 50.0), 50),
         layer(delta(4, 1, 12, 20, 6), None),
+        layer(latent(2, 16, 8, 12, 320, 0.25), None),       # a latent wider than the matrix-core kernels take
     ],
 }
 
