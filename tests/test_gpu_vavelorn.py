@@ -149,6 +149,31 @@ def test_a_wider_model_through_the_prompt_kernels(models, dtype):
     assert_close(np.concatenate([head, feed(stepper, "c", tokens[580:], [1])]), expected, dtype, "W decoded alone")
 
 
+def test_a_long_prompt_whole_and_in_portions(models):
+    """3,000 tokens of the wider model (47 pages, twenty chunks, far keys over the latent): in one step, and in
+    portions of 1,000, 513, 1,300 and 7 tokens with the last 100 decoded one by one. float32: the same bits; bfloat16:
+    the same to rounding."""
+    from flyweight_amd.engine import StepEntry
+    tokens = random_tokens(CONFIGS["W"]["vocab"], 3000, seed=12)
+    for dtype in DTYPES:
+        loaded = models("W", dtype)
+        stepper = loaded.stepper(num_pages=48, max_requests=2)
+        stepper.admit("whole")
+        whole = stepper.step([StepEntry("whole", tokens, list(range(2900, 3000)))]).float().cpu().numpy()
+        stepper.release("whole")
+        stepper.admit("cut")
+        at = 0
+        for n in (1000, 513, 1300, 7, 80):
+            stepper.step([StepEntry("cut", tokens[at:at + n], [n - 1])])
+            at += n
+        assert at == 2900
+        tail = np.concatenate([stepper.step([StepEntry("cut", [token], [0])]).float().cpu().numpy() for token in tokens[2900:]])
+        if dtype == "float32":
+            assert np.array_equal(tail, whole)
+        else:
+            assert np.abs(tail - whole).max() <= 0.05 * np.abs(whole).max()
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("variant", ["attention", "latent_attention", "delta"])
 @pytest.mark.parametrize("name", ["X", "Y"])
