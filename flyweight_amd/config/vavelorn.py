@@ -50,6 +50,16 @@ def _number(data, key, where, positive=False) -> float:
     return float(value)
 
 
+def _or(data, key, where, default, least=1) -> int:
+    """A size that may be left out: kv_heads (then every head has keys of its own), vdim (then the keys' size)."""
+    return _int(data, key, where, least) if isinstance(data, Mapping) and data.get(key) is not None else default
+
+
+def _scale(data, where, dim: int) -> float:
+    """The factor on the scores; left out, dim^-1/2."""
+    return _number(data, "scale", where, positive=True) if data.get("scale") is not None else dim ** -0.5
+
+
 def _groups(heads: int, kv_heads: int, where: str) -> None:
     if heads % kv_heads:
         raise ConfigError(f"config.json: {where}: {heads} heads are not a multiple of {kv_heads} kv_heads")
@@ -72,8 +82,9 @@ class ChunkedAttentionSizes:
     @classmethod
     def from_dict(cls, data, where) -> "ChunkedAttentionSizes":
         rot, mask, cap = data.get("rot"), data.get("mask"), data.get("softcap")
-        sizes = cls(heads=_int(data, "heads", where), kv_heads=_int(data, "kv_heads", where), dim=_int(data, "dim", where),
-                    vdim=_int(data, "vdim", where), scale=_number(data, "scale", where, positive=True),
+        heads, dim = _int(data, "heads", where), _int(data, "dim", where)
+        sizes = cls(heads=heads, kv_heads=_or(data, "kv_heads", where, heads), dim=dim,
+                    vdim=_or(data, "vdim", where, dim), scale=_scale(data, where, dim),
                     chunk=_int(mask, "size", where + ".mask") if mask is not None else None,
                     softcap=_number(data, "softcap", where, positive=True) if cap else None,
                     rot_dims=_int(rot, "dims", where + ".rot", least=0) if rot is not None else 0,
@@ -106,9 +117,9 @@ class LatentAttentionSizes:
 
     @classmethod
     def from_dict(cls, data, where) -> "LatentAttentionSizes":
-        return cls(heads=_int(data, "heads", where), dim=_int(data, "dim", where), vdim=_int(data, "vdim", where),
-                   q_rank=_int(data, "q_rank", where), kv_rank=_int(data, "kv_rank", where),
-                   scale=_number(data, "scale", where, positive=True))
+        dim = _int(data, "dim", where)
+        return cls(heads=_int(data, "heads", where), dim=dim, vdim=_or(data, "vdim", where, dim),
+                   q_rank=_int(data, "q_rank", where), kv_rank=_int(data, "kv_rank", where), scale=_scale(data, where, dim))
 
     def to_dict(self) -> Dict[str, Any]:
         return {"dim": self.dim, "heads": self.heads, "kv_rank": self.kv_rank, "q_rank": self.q_rank, "scale": self.scale,
@@ -127,8 +138,9 @@ class DeltaSizes:
 
     @classmethod
     def from_dict(cls, data, where) -> "DeltaSizes":
-        sizes = cls(heads=_int(data, "heads", where), kv_heads=_int(data, "kv_heads", where), dim=_int(data, "dim", where),
-                    vdim=_int(data, "vdim", where), conv=_int(data, "conv", where))
+        heads, dim = _int(data, "heads", where), _int(data, "dim", where)
+        sizes = cls(heads=heads, kv_heads=_or(data, "kv_heads", where, heads), dim=dim, vdim=_or(data, "vdim", where, dim),
+                    conv=_int(data, "conv", where))
         _groups(sizes.heads, sizes.kv_heads, where)
         return sizes
 
